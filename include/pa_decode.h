@@ -1,0 +1,156 @@
+/*
+ * pa_decode.h -- C ABI of the MI355X (gfx950) split-KV paged-attention decode library.
+ *
+ * The reference exposes this path as a Python function that launches Triton/Gluon kernels
+ * (pa_decode_triton_gluon_fp8.py:1659-1897 `paged_attention_decode`, twin
+ * pa_decode_triton.py:523-685); it has no C interface of its own.  The entry points below are
+ * what a foreign-function binding for that path binds instead: plain device pointers, element
+ * strides exactly as the reference passes them to its kernels
+ * (pa_decode_triton_gluon_fp8.py:1822-1841), sizes, enums, and a HIP stream handle.
+ *
+ * All functions return 0 on success or a negative PA_ERR_* code; none throws, allocates device
+ * memory, synchronises the host with the device, or keeps a pointer after it returns.  All
+ * kernels are enqueued on the given stream.  The library is re-entrant.
+ */
+#ifndef PA_DECODE_H_
+#define PA_DECODE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PA_DECODE_ABI_VERSION 1
+
+/* element types */
+enum { PA_DTYPE_BF16 = 0, PA_DTYPE_FP8_E4M3FN = 1 };
+/* quantisation modes, numbered as the reference numbers them
+ * (pa_decode_triton_gluon_fp8.py:1753-1790): -1 no scale, 0 one f32 per tensor (read from
+ * device memory), 1 one f32 per token and kv-head ([num_blocks, num_kv_heads, block_size, 1]) */
+enum { PA_QUANT_NONE = -1, PA_QUANT_PER_TENSOR = 0, PA_QUANT_PER_TOKEN = 1 };
+
+enum {
+  PA_OK = 0,
+  PA_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+  PA_ERR_BAD_STRUCT = -2,     /* struct_size does not match this library */
+  PA_ERR_UNSUPPORTED = -3,    /* dtype / head size / block size / group size not supported */
+  PA_ERR_BAD_SHAPE = -4,      /* non-positive size, bad partition size, stride the kernels cannot take */
+  PA_ERR_LAUNCH = -5,         /* the HIP runtime refused the launch (see pa_decode_last_hip_error) */
+  PA_ERR_NO_DEVICE = -6
+};
+
+/*
+ * Arguments of one decode call.  Shapes (B = num_seqs, Hkv = num_kv_heads, G = group_size
+ * = query heads per kv head, q = q_len, Ge = q*G, D = head_size, bs = block_size,
+ * P = max_num_partitions, x = 16 / sizeof(kv element)):
+ *
+ *   output        bf16 [B, Hkv*Ge, D]      row of (kv head h, new token t, head g) = h*Ge + t*G + g
+ *   query         bf16 or fp8 [B, Hkv*Ge, D]   same row order
+ *   key_cache     [num_blocks, Hkv, D/x, bs, x]
+ *   value_cache   [num_blocks, Hkv, D, bs]           (v_transposed = 0)
+ *                 [num_blocks, Hkv, bs/x, D, x]      (v_transposed = 1)
+ *   context_lens  int32 [B]   tokens in the cache for each sequence, the q new ones included
+ *   block_tables  int32 [B, >= ceil(ctx/bs)]
+ *   q_lens        int32 [B] or NULL: per-sequence number of new tokens (1..q); rows t >= q_lens[b]
+ *                 are padding and their output rows are written as zero
+ *   exp_sums, max_logits   f32 [B, Hkv, P, Ge]
+ *   tmp_output             bf16 [B, Hkv, P, Ge, D]
+ *
+ * Strides are in elements.  The innermost dimension of every tensor must be contiguous; for the
+ * caches the two innermost ones ([bs, x] of K, [bs] of V, [D, x] of transposed V) must be dense.
+ */
+typedef struct PaDecodeArgs {
+  uint32_t struct_size; /* = sizeof(PaDecodeArgs) */
+  int32_t reserved0;
+
+  void* output;
+  const void* query;
+  const void* key_cache;
+  const void* value_cache;
+  const int32_t* context_lens;
+  const int32_t* block_tables;
+  const int32_t* q_lens;      /* optional */
+  const float* query_scale;   /* optional; per tensor: 1 value, per token: [B, Hkv*Ge, 1] */
+  const float* key_scale;     /* optional */
+  const float* value_scale;   /* optional */
+  const float* alibi_slopes;  /* optional, [Hkv*G] */
+  float* exp_sums;
+  float* max_logits;
+  void* tmp_output;
+
+  int32_t num_seqs;
+  int32_t num_kv_heads;
+  int32_t group_size;          /* G */
+  int32_t q_len;               /* q (the maximum over the batch when q_lens is given) */
+  int32_t head_size;           /* D, 128 */
+  int32_t block_size;          /* 16, 64 or 1024 */
+  int32_t max_num_partitions;  /* P: partition axis length of the three buffers */
+  int32_t partition_size;      /* tokens per partition, a multiple of 256 */
+  int32_t query_dtype;         /* PA_DTYPE_* */
+  int32_t kv_dtype;            /* PA_DTYPE_* */
+  int32_t query_quant_mode;    /* PA_QUANT_* */
+  int32_t kv_quant_mode;       /* PA_QUANT_* */
+  int32_t v_transposed;
+  float softmax_scale;
+
+  int64_t stride_out_s, stride_out_h;
+  int64_t stride_q_s, stride_q_h;
+  int64_t stride_k_b, stride_k_h, stride_k_c;     /* block, kv head, 16-byte chunk row */
+  int64_t stride_v_b, stride_v_h, stride_v_2;     /* block, kv head, dim 2 (D rows, or bs/x rows) */
+  int64_t stride_bt_s;
+  int64_t stride_es_s, stride_es_h, stride_es_p;  /* shared by exp_sums and max_logits */
+  int64_t stride_tmp_s, stride_tmp_h, stride_tmp_p, stride_tmp_g;
+  int64_t stride_qscale_s;                        /* per-token query scale: stride of dim 0 */
+  int64_t stride_kvscale_b, stride_kvscale_h;     /* per-token kv scales: block, kv head */
+} PaDecodeArgs;
+
+/* Library / ABI identification. */
+int pa_decode_abi_version(void);
+uint32_t pa_decode_args_size(void);
+const char* pa_decode_error_string(int code);
+/* hipError_t of the last failed launch on the calling thread (0 if none). */
+int pa_decode_last_hip_error(void);
+
+/*
+ * Launch-time tuning layer; replaces the constants and the 15 lines of kernel selection in
+ * pa_decode_triton_gluon_fp8.py:24,1492-1509,1563-1564.  Given the batch shape and the longest
+ * context, returns the partition size (a multiple of 256) the partition kernel should use.
+ * Pure host arithmetic; num_cus <= 0 means "ask the current device".
+ */
+int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int32_t rows_per_group,
+                                    int32_t max_context_len, int32_t block_size, int32_t num_cus);
+
+/*
+ * Stage 1: one (sequence, kv head, partition) per wave.  Gathers the partition's KV pages through
+ * block_tables, computes softmax(scale * Q K^T + mask) V over the partition on MFMA and writes
+ * max_logits (max of the scaled logits), exp_sums (un-normalised) and tmp_output (normalised).
+ * Replaces paged_attention_decode_v2_gluon_fp8 / _large_block_fp8
+ * (pa_decode_triton_gluon_fp8.py:514-1002, :27-501) and
+ * _paged_attn_decode_v2_w_dot_kernel_reshape_noloop_qk (pa_decode_triton.py:26-224).
+ * Partitions at or beyond ceil(context_len / partition_size) are not written.
+ */
+int pa_decode_partition(const PaDecodeArgs* args, void* hip_stream);
+
+/*
+ * Stage 2: merges the first ceil(context_len / partition_size) partitions of every row into
+ * output.  Replaces paged_attention_decode_v2_reduce_kernel
+ * (pa_decode_triton_gluon_fp8.py:1187-1333) and _paged_attn_decode_v2_w_dot_reduce_kernel
+ * (pa_decode_triton.py:227-324).
+ */
+int pa_decode_reduce(const PaDecodeArgs* args, void* hip_stream);
+
+/* Both stages back to back on one stream: the body of the reference's paged_attention_decode. */
+int pa_decode(const PaDecodeArgs* args, void* hip_stream);
+
+/*
+ * Test hook: decodes n FP8 e4m3fn bytes (device pointer) to f32 (device pointer) with the same
+ * conversion instructions the partition kernel uses, so the dequantisation table can be compared
+ * with the format definition code by code.
+ */
+int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PA_DECODE_H_ */

@@ -1,0 +1,98 @@
+"""ctypes binding of libpa_decode.so (the C ABI in include/pa_decode.h).
+
+The library is loaded lazily and never built here: a missing library is an error, not a reason
+to fall back to another implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libpa_decode.so")
+
+PA_DECODE_ABI_VERSION = 1
+PA_DTYPE_BF16, PA_DTYPE_FP8_E4M3FN = 0, 1
+PA_QUANT_NONE, PA_QUANT_PER_TENSOR, PA_QUANT_PER_TOKEN = -1, 0, 1
+
+EXPORTED_SYMBOLS = (
+    "pa_decode_abi_version",
+    "pa_decode_args_size",
+    "pa_decode_error_string",
+    "pa_decode_last_hip_error",
+    "pa_decode_select_partition_size",
+    "pa_decode_partition",
+    "pa_decode_reduce",
+    "pa_decode",
+    "pa_debug_fp8_decode",
+)
+
+
+class PaDecodeArgs(C.Structure):
+    _fields_ = (
+        [("struct_size", C.c_uint32), ("reserved0", C.c_int32)]
+        + [(n, C.c_void_p) for n in (
+            "output", "query", "key_cache", "value_cache", "context_lens", "block_tables", "q_lens",
+            "query_scale", "key_scale", "value_scale", "alibi_slopes", "exp_sums", "max_logits", "tmp_output")]
+        + [(n, C.c_int32) for n in (
+            "num_seqs", "num_kv_heads", "group_size", "q_len", "head_size", "block_size",
+            "max_num_partitions", "partition_size", "query_dtype", "kv_dtype", "query_quant_mode",
+            "kv_quant_mode", "v_transposed")]
+        + [("softmax_scale", C.c_float)]
+        + [(n, C.c_int64) for n in (
+            "stride_out_s", "stride_out_h", "stride_q_s", "stride_q_h",
+            "stride_k_b", "stride_k_h", "stride_k_c", "stride_v_b", "stride_v_h", "stride_v_2",
+            "stride_bt_s", "stride_es_s", "stride_es_h", "stride_es_p",
+            "stride_tmp_s", "stride_tmp_h", "stride_tmp_p", "stride_tmp_g",
+            "stride_qscale_s", "stride_kvscale_b", "stride_kvscale_h")]
+    )
+
+
+class PaDecodeLibraryError(RuntimeError):
+    pass
+
+
+_lib = None
+_lock = threading.Lock()
+
+
+def load_library(path: str = LIB_PATH) -> C.CDLL:
+    """dlopen the HIP library and check that its struct layout matches this binding."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(path):
+            raise PaDecodeLibraryError(
+                f"{path} is missing: build it with `python -m triton_op_amd.build` "
+                "(there is no fallback implementation)")
+        lib = C.CDLL(path)
+        lib.pa_decode_abi_version.restype = C.c_int
+        lib.pa_decode_args_size.restype = C.c_uint32
+        lib.pa_decode_error_string.restype = C.c_char_p
+        lib.pa_decode_error_string.argtypes = [C.c_int]
+        lib.pa_decode_last_hip_error.restype = C.c_int
+        lib.pa_decode_select_partition_size.restype = C.c_int
+        lib.pa_decode_select_partition_size.argtypes = [C.c_int32] * 6
+        for name in ("pa_decode_partition", "pa_decode_reduce", "pa_decode"):
+            fn = getattr(lib, name)
+            fn.restype = C.c_int
+            fn.argtypes = [C.POINTER(PaDecodeArgs), C.c_void_p]
+        lib.pa_debug_fp8_decode.restype = C.c_int
+        lib.pa_debug_fp8_decode.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
+        if lib.pa_decode_abi_version() != PA_DECODE_ABI_VERSION:
+            raise PaDecodeLibraryError("libpa_decode.so has a different ABI version; rebuild it")
+        if lib.pa_decode_args_size() != C.sizeof(PaDecodeArgs):
+            raise PaDecodeLibraryError(
+                f"PaDecodeArgs is {lib.pa_decode_args_size()} bytes in the library but "
+                f"{C.sizeof(PaDecodeArgs)} in the binding")
+        _lib = lib
+        return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        lib = load_library()
+        msg = lib.pa_decode_error_string(rc).decode()
+        raise PaDecodeLibraryError(f"{what} failed: {msg} (code {rc}, hipError {lib.pa_decode_last_hip_error()})")

@@ -1,0 +1,61 @@
+"""Builds the HIP shared library of the decode op, in-tree, for gfx950.
+
+    python -m triton_op_amd.build
+
+`hipcc` cross-compiles without a GPU.  The result is triton_op_amd/libpa_decode.so, which the
+ctypes binding in `_cabi.py` loads; nothing is JIT-compiled at import or call time.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SOURCES = [os.path.join(HERE, "csrc", "pa_decode.hip")]
+HEADERS = [os.path.join(HERE, "..", "include", "pa_decode.h")]
+LIB_PATH = os.path.join(HERE, "libpa_decode.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fno-strict-aliasing",
+    "-fPIC",
+    "-shared",
+    # packed-FP32 VALU forms are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def find_hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or put /opt/rocm/bin on PATH)")
+
+
+def build(verbose: bool = True, extra_flags=()) -> str:
+    cmd = [find_hipcc(), *HIPCC_FLAGS, *extra_flags, *SOURCES, "-o", LIB_PATH]
+    if verbose:
+        print("[triton_op_amd.build]", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass warns that it does not know the packed-fp32-ops feature; that is expected
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return LIB_PATH
+
+
+def is_stale() -> bool:
+    if not os.path.exists(LIB_PATH):
+        return True
+    t = os.path.getmtime(LIB_PATH)
+    return any(os.path.getmtime(p) > t for p in SOURCES + HEADERS)
+
+
+if __name__ == "__main__":
+    build()

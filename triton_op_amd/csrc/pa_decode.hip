@@ -1,0 +1,763 @@
+// Split-KV paged-attention decode for MI355X (gfx950 / CDNA4): partition kernel, reduce kernel
+// and the C ABI declared in include/pa_decode.h.
+//
+// Work decomposition.  One wavefront (64 lanes) owns one (sequence, kv head, partition) and keeps
+// private online-softmax state (m, l, O); nothing is shared between waves, so there are no
+// workgroup barriers.  A partition is walked in steps of 64 tokens (four 16-token tiles):
+//
+//   K tile  (16 tokens x 128 dims): every lane loads 16 bytes = one [token][16-byte chunk] cell of
+//           the cache; lanes 0-15 are the 16 tokens of a page, lane>>4 picks the chunk row, so a
+//           wave load covers 4 x 256 contiguous bytes in storage order.  The 16 bytes are the A
+//           operand of two 16x16x32 MFMA k-steps (the dot product does not care in which order the
+//           head dimension is summed, so the query operand is loaded in the matching order).
+//   S^T = K Q^T on v_mfma_f32_16x16x32_bf16: tokens are the M rows, query rows (GQA group x MTP
+//           position, padded to 16) are the N columns, so a lane ends up with 4 tokens of ONE
+//           query row and the softmax max/sum need only two cross-lane steps (lane^16, lane^32).
+//   P       goes through a wave-private LDS tile to become the B operand of the second MFMA.
+//   V tile  (128 dims x 16 tokens): every lane loads 16 bytes = 16 tokens of one head dim, lanes
+//           0-15 are 16 consecutive dims (256 contiguous bytes), lane>>4 picks one of the four
+//           tiles of the step.  O^T = V^T P^T accumulates in 8 MFMA tiles of [16 dims x 16 rows].
+//
+// FP8 e4m3fn is widened to bf16 exactly (3 mantissa bits fit in 7); per-tensor scales are folded
+// into the softmax scale (K) and the epilogue (V), per-token scales multiply S and P in f32.
+// The next step's K/V/page ids are in flight while the current step is computed.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/pa_decode.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr int kHeadSize = 128;
+constexpr int kStepTokens = 64;     // tokens per pipeline step (4 tiles of 16)
+constexpr int kChunkTokens = 256;   // page ids are fetched for 256 tokens (4 steps) at a time
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kPRowBytes = 144;     // 64 tokens * 2 B + 16 B pad per query row of the P tile
+
+union Bf16x8Bits {
+  bf16x8 v;
+  bf16x2 p[4];
+  u32x4 u;
+};
+
+// two FP8 e4m3fn bytes -> two f32 (v_cvt_pk_f32_fp8), then keep the upper 16 bits of each:
+// exact, since an e4m3 value has 3 mantissa bits and bf16 keeps 7.
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t word, bool high_half) {
+  f32x2 f = high_half ? __builtin_amdgcn_cvt_pk_f32_fp8((int)word, true)
+                      : __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
+  return __builtin_amdgcn_perm(__float_as_uint(f[1]), __float_as_uint(f[0]), 0x07060302u);
+}
+
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t lo, uint32_t hi) {
+  Bf16x8Bits r;
+  r.u[0] = fp8x2_to_bf16x2(lo, false);
+  r.u[1] = fp8x2_to_bf16x2(lo, true);
+  r.u[2] = fp8x2_to_bf16x2(hi, false);
+  r.u[3] = fp8x2_to_bf16x2(hi, true);
+  return r.v;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  union {
+    bf16x2 v;
+    uint32_t u;
+  } r;
+  r.v[0] = (__bf16)a;
+  r.v[1] = (__bf16)b;
+  return r.u;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// keep the first `n` (0..16) bytes of a 16-byte vector, zero the rest
+__device__ __forceinline__ u32x4 keep_first_bytes(u32x4 v, int n) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    int k = n - 4 * w;
+    uint32_t m = k >= 4 ? 0xffffffffu : (k <= 0 ? 0u : ((1u << (8 * k)) - 1u));
+    v[w] &= m;
+  }
+  return v;
+}
+
+// One step's worth of cache data, as loaded (still FP8 / bf16 bit patterns).
+template <int KVT, bool PER_TOKEN>
+struct StepData {
+  static constexpr int NKL = KVT == PA_DTYPE_FP8_E4M3FN ? 2 : 4;  // 16-byte K loads per lane per tile
+  static constexpr int NVL = KVT == PA_DTYPE_FP8_E4M3FN ? 1 : 2;  // 16-byte V loads per lane per 16 dims
+  u32x4 k[4][NKL];
+  u32x4 v[8][NVL];
+  f32x4 ks[PER_TOKEN ? 4 : 1];
+  f32x4 vs[PER_TOKEN ? 4 : 1];
+};
+
+struct WaveCtx {
+  const char* kbase;   // key_cache + head offset (bytes)
+  const char* vbase;   // value_cache + head offset (bytes)
+  const float* ksbase; // key_scale + head offset
+  const float* vsbase;
+  int64_t k_block_bytes, v_block_bytes, kvs_block;
+  uint32_t k_lane_off[4];  // per-lane byte offset of K load ld inside a tile
+  uint32_t v_row_bytes;    // byte distance between consecutive head dims of V
+  uint32_t v_half_bytes;   // byte distance between the two 8-token halves of a bf16 V tile
+  int log2_bs;
+  int bs_mask;
+  int v_transposed;
+  int64_t v_group_bytes;   // transposed V: bytes between consecutive 16-token tiles of a page
+};
+
+// page id of the 16-token tile `tile` (uniform value broadcast from the page-id register)
+__device__ __forceinline__ int tile_page(const int* pages4, int step_in_chunk, int j) {
+  return __builtin_amdgcn_readlane(pages4[step_in_chunk], 16 * j);
+}
+
+template <int KVT, bool PER_TOKEN>
+__device__ __forceinline__ void load_step(StepData<KVT, PER_TOKEN>& sd, const WaveCtx& c, int page_lane,
+                                          int tok0, int first_tile_tok, int last_tile_tok, int li, int kg,
+                                          int esz) {
+  // K: tile j of the step, same page for the whole wave
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int t = tok0 + 16 * j;
+    t = t > last_tile_tok ? last_tile_tok : t;
+    int page = __builtin_amdgcn_readlane(page_lane, 16 * j);
+    const char* tb = c.kbase + (int64_t)page * c.k_block_bytes + (int64_t)(t & c.bs_mask) * 16;
+#pragma unroll
+    for (int ld = 0; ld < StepData<KVT, PER_TOKEN>::NKL; ++ld) sd.k[j][ld] = load16(tb + c.k_lane_off[ld]);
+    if constexpr (PER_TOKEN) {
+      const float* sb = c.ksbase + (int64_t)page * c.kvs_block + (t & c.bs_mask) + 4 * kg;
+      sd.ks[j] = *reinterpret_cast<const f32x4*>(sb);
+      const float* vb = c.vsbase + (int64_t)page * c.kvs_block + (t & c.bs_mask) + 4 * kg;
+      sd.vs[j] = *reinterpret_cast<const f32x4*>(vb);
+    }
+  }
+  // V: lane group kg owns tile kg of the step
+  {
+    int t = tok0 + 16 * kg;
+    t = t > last_tile_tok ? last_tile_tok : t;
+    int off = t & c.bs_mask;
+    const char* tb = c.vbase + (int64_t)page_lane * c.v_block_bytes +
+                     (c.v_transposed ? (int64_t)(off >> 4) * c.v_group_bytes : (int64_t)off * esz);
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const char* rp = tb + (uint32_t)(16 * db + li) * c.v_row_bytes;
+#pragma unroll
+      for (int hf = 0; hf < StepData<KVT, PER_TOKEN>::NVL; ++hf) sd.v[db][hf] = load16(rp + hf * c.v_half_bytes);
+    }
+  }
+  (void)first_tile_tok;
+}
+
+template <int NT>
+struct RowState {
+  float m[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
+  float l[NT];      // this lane's share of the running sum of exp2(s - m)
+  f32x4 acc[NT][8]; // O^T: [16*db + 4*kg + r][row]
+};
+
+// DEPTH 2 keeps the next step's loads in flight during the current step's arithmetic (two register
+// copies of a step's cache data); DEPTH 1 loads and computes in turn and leaves the overlap to the
+// other waves of the SIMD.  OCC is the number of waves per SIMD the register budget is cut for.
+template <int NT, int KVT, bool PER_TOKEN, int WAVES, int DEPTH, int OCC>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void pa_partition_kernel(const PaDecodeArgs a) {
+  constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
+  constexpr int esz = kFp8 ? 1 : 2;
+  typedef StepData<KVT, PER_TOKEN> SD;
+
+  __shared__ __attribute__((aligned(16))) char p_lds[WAVES][NT][16 * kPRowBytes];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int li = lane & 15;
+  const int kg = lane >> 4;
+
+  // ---- which (sequence, head, partition) -------------------------------------------------
+  const int P = a.max_num_partitions;
+  const int Hkv = a.num_kv_heads;
+  const long long wid = (long long)blockIdx.x * WAVES + wave;
+  const long long total = (long long)a.num_seqs * P * Hkv;
+  if (wid >= total) return;
+  const int h = (int)(wid % Hkv);
+  const int part = (int)((wid / Hkv) % P);
+  const int b = (int)(wid / ((long long)Hkv * P));
+
+  const int ctx = a.context_lens[b];
+  const int part_start = part * a.partition_size;
+  if (part_start >= ctx) return;
+  const int part_end = min(part_start + a.partition_size, ctx);
+  const int G = a.group_size;
+  const int Ge = a.q_len * G;  // rows per kv head in the buffers
+  const int qb = a.q_lens ? a.q_lens[b] : a.q_len;
+  const int rows_valid = qb * G;
+
+  // ---- per-lane row bookkeeping -----------------------------------------------------------
+  int limit[NT];      // number of visible keys of this lane's query row
+  float slope2[NT];   // ALiBi slope * log2e
+  const bool has_alibi = a.alibi_slopes != nullptr;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int row = 16 * nt + li;
+    int t = row / G;
+    limit[nt] = row < rows_valid ? ctx - (qb - 1 - t) : 0;
+    slope2[nt] = (has_alibi && row < rows_valid) ? a.alibi_slopes[h * G + (row - t * G)] * kLog2e : 0.f;
+  }
+  const int min_limit = ctx - (qb - 1);  // keys below this index are visible to every real row
+
+  // ---- query: B operand of S^T = K Q^T ------------------------------------------------------
+  // k-step s of a tile covers, for lane group kg, the 8 head dims the K load puts in that slot.
+  bf16x8 qreg[NT][4];
+  {
+    const char* qb_ptr = (const char*)a.query;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      int row = 16 * nt + li;
+      bool ok = row < rows_valid;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
+        Bf16x8Bits q;
+        q.u = u32x4{0, 0, 0, 0};
+        if (ok) {
+          int64_t e = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + row) * a.stride_q_h + dim;
+          if (a.query_dtype == PA_DTYPE_BF16) {
+            q.u = load16(qb_ptr + e * 2);
+          } else {
+            u32x2 raw = *reinterpret_cast<const u32x2*>(qb_ptr + e);
+            q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
+          }
+        }
+        qreg[nt][s] = q.v;
+      }
+    }
+  }
+  // per-row query scale (FP8 query) multiplies the logits of that row
+  float qscale[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int row = 16 * nt + li;
+    qscale[nt] = 1.f;
+    if (a.query_quant_mode == PA_QUANT_PER_TENSOR) qscale[nt] = a.query_scale[0];
+    if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row < rows_valid)
+      qscale[nt] = a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
+  }
+
+  // ---- cache addressing ---------------------------------------------------------------------
+  WaveCtx c;
+  c.log2_bs = 31 - __builtin_clz(a.block_size);
+  c.bs_mask = a.block_size - 1;
+  c.kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h * esz;
+  c.vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h * esz;
+  c.k_block_bytes = a.stride_k_b * esz;
+  c.v_block_bytes = a.stride_v_b * esz;
+  c.kvs_block = a.stride_kvscale_b;
+  c.ksbase = PER_TOKEN ? a.key_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  c.vsbase = PER_TOKEN ? a.value_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+#pragma unroll
+  for (int ld = 0; ld < 4; ++ld) c.k_lane_off[ld] = (uint32_t)((4 * ld + kg) * a.stride_k_c * esz + li * 16);
+  c.v_transposed = a.v_transposed;
+  if (a.v_transposed) {
+    c.v_row_bytes = 16;
+    c.v_group_bytes = a.stride_v_2 * esz * esz;  // a 16-token tile is 16/x = esz groups of x tokens
+    c.v_half_bytes = (uint32_t)(a.stride_v_2 * esz);
+  } else {
+    c.v_row_bytes = (uint32_t)(a.stride_v_2 * esz);
+    c.v_group_bytes = 0;
+    c.v_half_bytes = 16;
+  }
+  float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
+  if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
+    k_tensor_scale = a.key_scale[0];
+    v_tensor_scale = a.value_scale[0];
+  }
+  const float scale2 = a.softmax_scale * k_tensor_scale * kLog2e;
+
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const int last_tile_tok = (part_end - 1) & ~15;  // first token of the last tile that holds a live token
+
+  // page ids: lane group kg keeps the page of tile (4*step + kg) for the 4 steps of a 256-token chunk
+  auto load_pages = [&](int chunk_tok0, int* pages4) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      int t = chunk_tok0 + kStepTokens * s + 16 * kg;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      pages4[s] = bt[t >> c.log2_bs];
+    }
+  };
+
+  RowState<NT> st;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    st.m[nt] = -INFINITY;
+    st.l[nt] = 0.f;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) st.acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  char* plds = &p_lds[wave][0][0];
+
+  // ---- one step of 64 tokens -------------------------------------------------------------------
+  auto compute_step = [&](SD& sd, int tok0) {
+    // S^T tiles
+    f32x4 s[NT][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) s[nt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ld = 0; ld < SD::NKL; ++ld) {
+        if constexpr (kFp8) {
+          bf16x8 a0 = fp8x8_to_bf16x8(sd.k[j][ld][0], sd.k[j][ld][1]);
+          bf16x8 a1 = fp8x8_to_bf16x8(sd.k[j][ld][2], sd.k[j][ld][3]);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[nt][2 * ld], s[nt][j], 0, 0, 0);
+            s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[nt][2 * ld + 1], s[nt][j], 0, 0, 0);
+          }
+        } else {
+          Bf16x8Bits ka;
+          ka.u = sd.k[j][ld];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka.v, qreg[nt][ld], s[nt][j], 0, 0, 0);
+        }
+      }
+    }
+
+    const bool full = (tok0 + kStepTokens <= min_limit) && !has_alibi;  // wave-uniform
+    if (!full) {
+      // zero the V bytes of tokens at or beyond ctx (stale cache contents may decode to NaN)
+      int nvalid = ctx - (tok0 + 16 * kg);
+      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        if constexpr (kFp8) {
+          sd.v[db][0] = keep_first_bytes(sd.v[db][0], nvalid);
+        } else {
+          sd.v[db][0] = keep_first_bytes(sd.v[db][0], 2 * (nvalid > 8 ? 8 : nvalid));
+          sd.v[db][1] = keep_first_bytes(sd.v[db][1], 2 * (nvalid > 8 ? nvalid - 8 : 0));
+        }
+      }
+    }
+
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float rs = scale2 * qscale[nt];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = s[nt][j][r] * rs;
+          if constexpr (PER_TOKEN) v *= sd.ks[j][r];
+          if (!full) {
+            int col = tok0 + 16 * j + 4 * kg + r;
+            v += slope2[nt] * (float)(col - ctx + 1);
+            v = col < limit[nt] ? v : -INFINITY;
+          }
+          s[nt][j][r] = v;
+          mx = fmaxf(mx, v);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(st.m[nt], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2(st.m[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
+      st.m[nt] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float p0 = fast_exp2(s[nt][j][0] - m_safe);
+        float p1 = fast_exp2(s[nt][j][1] - m_safe);
+        float p2 = fast_exp2(s[nt][j][2] - m_safe);
+        float p3 = fast_exp2(s[nt][j][3] - m_safe);
+        psum += (p0 + p1) + (p2 + p3);
+        if constexpr (PER_TOKEN) {
+          // a masked token's scale may be stale memory (NaN): its weight must stay exactly 0
+          f32x4 vsc = sd.vs[j];
+          if (!full) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vsc[r] = s[nt][j][r] == -INFINITY ? 0.f : vsc[r];
+          }
+          p0 *= vsc[0];
+          p1 *= vsc[1];
+          p2 *= vsc[2];
+          p3 *= vsc[3];
+        }
+        u32x2 pk;
+        pk[0] = pack_bf16x2(p0, p1);
+        pk[1] = pack_bf16x2(p2, p3);
+        *reinterpret_cast<u32x2*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes + (16 * j + 4 * kg) * 2) = pk;
+      }
+      st.l[nt] = st.l[nt] * alpha + psum;
+#pragma unroll
+      for (int db = 0; db < 8; ++db) st.acc[nt][db] *= alpha;
+    }
+
+    // the P tile is written and read by this wave only; LDS operations of one wave complete in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // O^T += V^T P^T
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      bf16x8 pb[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        Bf16x8Bits t;
+        t.u = *reinterpret_cast<const u32x4*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes +
+                                              (16 * kg + 8 * hf) * 2);
+        pb[nt] = t.v;
+      }
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        bf16x8 va;
+        if constexpr (kFp8) {
+          va = fp8x8_to_bf16x8(sd.v[db][0][2 * hf], sd.v[db][0][2 * hf + 1]);
+        } else {
+          Bf16x8Bits t;
+          t.u = sd.v[db][hf];
+          va = t.v;
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          st.acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nt], st.acc[nt][db], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---- main loop: chunks of 256 tokens, 4 steps each, next step's data in flight -------------------
+  const int n_steps = (part_end - part_start + kStepTokens - 1) / kStepTokens;
+  int pages_cur[4], pages_next[4];
+  load_pages(part_start, pages_cur);
+  SD buf0, buf1;
+  load_step<KVT, PER_TOKEN>(buf0, c, pages_cur[0], part_start, part_start, last_tile_tok, li, kg, esz);
+
+  int step = 0;
+  for (int chunk_tok0 = part_start; chunk_tok0 < part_end; chunk_tok0 += kChunkTokens) {
+    const bool more_chunks = chunk_tok0 + kChunkTokens < part_end;
+    if (more_chunks) load_pages(chunk_tok0 + kChunkTokens, pages_next);
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const int tok0 = chunk_tok0 + kStepTokens * s4;
+      if (step < n_steps) {  // wave-uniform
+        const bool has_next = step + 1 < n_steps;
+        const int np = s4 < 3 ? pages_cur[s4 + 1] : pages_next[0];
+        if constexpr (DEPTH == 2) {
+          SD& cur = (s4 & 1) ? buf1 : buf0;
+          SD& nxt = (s4 & 1) ? buf0 : buf1;
+          if (has_next)
+            load_step<KVT, PER_TOKEN>(nxt, c, np, tok0 + kStepTokens, part_start, last_tile_tok, li, kg, esz);
+          compute_step(cur, tok0);
+        } else {
+          compute_step(buf0, tok0);
+          if (has_next)
+            load_step<KVT, PER_TOKEN>(buf0, c, np, tok0 + kStepTokens, part_start, last_tile_tok, li, kg, esz);
+        }
+      }
+      ++step;
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) pages_cur[s] = pages_next[s];
+  }
+
+  // ---- epilogue: normalise, store m (natural-log domain), l and the bf16 partial output -----------
+  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+  char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                     (int64_t)part * a.stride_tmp_p) * 2;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float l = st.l[nt];
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    const int row = 16 * nt + li;
+    float m_out = st.m[nt] * (1.0f / kLog2e);
+    if (row >= rows_valid) {  // padding rows of a ragged batch: no visible key
+      l = 0.f;
+      m_out = -INFINITY;
+    }
+    const float inv = l > 0.f ? v_tensor_scale / l : 0.f;
+    if (row < Ge) {
+      if (kg == 0) {
+        a.max_logits[es_off + row] = m_out;
+        a.exp_sums[es_off + row] = l;
+      }
+      char* rp = tmp + (int64_t)row * a.stride_tmp_g * 2;
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        f32x4 o = st.acc[nt][db] * inv;
+        u32x2 pk;
+        pk[0] = pack_bf16x2(o[0], o[1]);
+        pk[1] = pack_bf16x2(o[2], o[3]);
+        *reinterpret_cast<u32x2*>(rp + (16 * db + 4 * kg) * 2) = pk;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// reduce: one wave per output row, two head dims per lane; streams over the partitions
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int Ge = a.q_len * a.group_size;
+  const long long rid = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long long total = (long long)a.num_seqs * a.num_kv_heads * Ge;
+  if (rid >= total) return;
+  const int row = (int)(rid % Ge);
+  const int h = (int)((rid / Ge) % a.num_kv_heads);
+  const int b = (int)(rid / ((long long)Ge * a.num_kv_heads));
+
+  const int ctx = a.context_lens[b];
+  int n = (ctx + a.partition_size - 1) / a.partition_size;
+  n = n > a.max_num_partitions ? a.max_num_partitions : n;
+  const int qb = a.q_lens ? a.q_lens[b] : a.q_len;
+
+  uint32_t* out = reinterpret_cast<uint32_t*>((char*)a.output +
+                                              ((int64_t)b * a.stride_out_s + (int64_t)(h * Ge + row) * a.stride_out_h) * 2) + lane;
+  if (n <= 0 || row >= qb * a.group_size) {
+    *out = 0u;
+    return;
+  }
+  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + row;
+  const float* ml = a.max_logits + es_off;
+  const float* es = a.exp_sums + es_off;
+  const char* tmp = (const char*)a.tmp_output +
+                    ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h + (int64_t)row * a.stride_tmp_g) * 2 +
+                    lane * 4;
+  const int64_t tp = a.stride_tmp_p * 2;
+
+  // global max over partitions
+  float M = -INFINITY;
+  for (int p = lane; p < n; p += 64) M = fmaxf(M, ml[(int64_t)p * a.stride_es_p]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  const float M_safe = M == -INFINITY ? 0.f : M;
+
+  float acc0 = 0.f, acc1 = 0.f, wsum = 0.f;
+  int p = 0;
+  for (; p + 4 <= n; p += 4) {
+    float w[4];
+    uint32_t t[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float m = ml[(int64_t)(p + u) * a.stride_es_p];
+      float l = es[(int64_t)(p + u) * a.stride_es_p];
+      w[u] = l > 0.f ? l * __expf(m - M_safe) : 0.f;
+      t[u] = *reinterpret_cast<const uint32_t*>(tmp + (int64_t)(p + u) * tp);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      wsum += w[u];
+      acc0 += bf16_bits_to_f32(t[u] & 0xffffu) * w[u];
+      acc1 += bf16_bits_to_f32(t[u] >> 16) * w[u];
+    }
+  }
+  for (; p < n; ++p) {
+    float m = ml[(int64_t)p * a.stride_es_p];
+    float l = es[(int64_t)p * a.stride_es_p];
+    float w = l > 0.f ? l * __expf(m - M_safe) : 0.f;
+    uint32_t t = *reinterpret_cast<const uint32_t*>(tmp + (int64_t)p * tp);
+    wsum += w;
+    acc0 += bf16_bits_to_f32(t & 0xffffu) * w;
+    acc1 += bf16_bits_to_f32(t >> 16) * w;
+  }
+  const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+  *out = pack_bf16x2(acc0 * inv, acc1 * inv);
+}
+
+__global__ void pa_fp8_decode_kernel(const uint8_t* codes, float* out, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  // same path as the partition kernel: byte -> bf16 bit pattern -> f32
+  uint32_t w = (uint32_t)codes[i] | ((uint32_t)codes[i] << 16);
+  uint32_t lo = fp8x2_to_bf16x2(w, false);
+  uint32_t hi = fp8x2_to_bf16x2(w, true);
+  float a = bf16_bits_to_f32(lo & 0xffffu);
+  float b = bf16_bits_to_f32(hi & 0xffffu);
+  out[i] = (i & 1) ? b : a;
+}
+
+thread_local int g_last_hip_error = 0;
+
+int check_common(const PaDecodeArgs* a) {
+  if (!a) return PA_ERR_NULL_POINTER;
+  if (a->struct_size != sizeof(PaDecodeArgs)) return PA_ERR_BAD_STRUCT;
+  if (!a->context_lens || !a->exp_sums || !a->max_logits || !a->tmp_output) return PA_ERR_NULL_POINTER;
+  if (a->num_seqs <= 0 || a->num_kv_heads <= 0 || a->group_size <= 0 || a->q_len <= 0 ||
+      a->max_num_partitions <= 0)
+    return PA_ERR_BAD_SHAPE;
+  if (a->partition_size <= 0 || a->partition_size % 256) return PA_ERR_BAD_SHAPE;
+  if (a->head_size != kHeadSize) return PA_ERR_UNSUPPORTED;
+  if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;
+  return PA_OK;
+}
+
+template <int NT, int KVT, bool PT>
+int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
+  constexpr int W = 1;
+  constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
+  constexpr int DEPTH = (NT == 1 && kFp8) ? 2 : 1;
+  constexpr int OCC = NT == 1 ? 2 : 1;
+  long long total = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
+  long long blocks = (total + W - 1) / W;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, W, DEPTH, OCC>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return PA_OK;
+}
+
+template <int KVT, bool PT>
+int launch_partition_nt(const PaDecodeArgs& a, int nt, hipStream_t stream) {
+  switch (nt) {
+    case 1: return launch_partition_w<1, KVT, PT>(a, stream);
+    case 2: return launch_partition_w<2, KVT, PT>(a, stream);
+    case 3:
+    case 4: return launch_partition_w<4, KVT, PT>(a, stream);
+  }
+  return PA_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pa_decode_abi_version(void) { return PA_DECODE_ABI_VERSION; }
+uint32_t pa_decode_args_size(void) { return (uint32_t)sizeof(PaDecodeArgs); }
+int pa_decode_last_hip_error(void) { return g_last_hip_error; }
+
+const char* pa_decode_error_string(int code) {
+  switch (code) {
+    case PA_OK: return "ok";
+    case PA_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case PA_ERR_BAD_STRUCT: return "PaDecodeArgs.struct_size does not match this library";
+    case PA_ERR_UNSUPPORTED: return "unsupported dtype, head size, block size or group size";
+    case PA_ERR_BAD_SHAPE: return "bad size, partition size or stride";
+    case PA_ERR_LAUNCH: return "HIP launch failed";
+    case PA_ERR_NO_DEVICE: return "no HIP device";
+  }
+  return "unknown error code";
+}
+
+int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int32_t rows_per_group,
+                                    int32_t max_context_len, int32_t block_size, int32_t num_cus) {
+  (void)rows_per_group;
+  (void)block_size;
+  if (num_seqs <= 0 || num_kv_heads <= 0 || max_context_len <= 0) return PA_ERR_BAD_SHAPE;
+  if (num_cus <= 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) num_cus = 256;
+    else num_cus = prop.multiProcessorCount;
+  }
+  // Enough waves to keep every SIMD busy several times over, as few partitions as that allows:
+  // each extra partition costs a (Ge x 128) bf16 partial written and read back.
+  const long long pairs = (long long)num_seqs * num_kv_heads;
+  const long long want_waves = (long long)num_cus * 4 * 6;
+  int part = 256;
+  while (part < 4096) {
+    long long parts_next = (max_context_len + 2 * part - 1) / (2 * part);
+    if (pairs * parts_next < want_waves) break;
+    part *= 2;
+  }
+  return part;
+}
+
+int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!a->query || !a->key_cache || !a->value_cache || !a->block_tables) return PA_ERR_NULL_POINTER;
+  if (a->block_size != 16 && a->block_size != 64 && a->block_size != 1024) return PA_ERR_UNSUPPORTED;
+  if (a->kv_dtype != PA_DTYPE_BF16 && a->kv_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
+  if (a->query_dtype != PA_DTYPE_BF16 && a->query_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
+  if (a->kv_quant_mode != PA_QUANT_NONE && (!a->key_scale || !a->value_scale)) return PA_ERR_NULL_POINTER;
+  if (a->query_quant_mode != PA_QUANT_NONE && !a->query_scale) return PA_ERR_NULL_POINTER;
+  if (a->kv_quant_mode < -1 || a->kv_quant_mode > 1 || a->query_quant_mode < -1 || a->query_quant_mode > 1)
+    return PA_ERR_UNSUPPORTED;
+  const int esz = a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
+  // 16-byte vector loads: every stride that moves a vector must keep it 16-byte aligned
+  if ((a->stride_k_b * esz) % 16 || (a->stride_k_h * esz) % 16 || (a->stride_k_c * esz) % 16 ||
+      (a->stride_v_b * esz) % 16 || (a->stride_v_h * esz) % 16 || (a->stride_v_2 * esz) % 16)
+    return PA_ERR_BAD_SHAPE;
+  const int qsz = a->query_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
+  if ((a->stride_q_s * qsz) % 16 || (a->stride_q_h * qsz) % 16) return PA_ERR_BAD_SHAPE;
+  if ((a->stride_tmp_g * 2) % 8 || (a->stride_tmp_p * 2) % 8 || (a->stride_tmp_h * 2) % 8 || (a->stride_tmp_s * 2) % 8)
+    return PA_ERR_BAD_SHAPE;
+  if (a->kv_quant_mode == PA_QUANT_PER_TOKEN && (a->stride_kvscale_b % 4 || a->stride_kvscale_h % 4))
+    return PA_ERR_BAD_SHAPE;
+  if ((long long)(4 * 3 + 3) * a->stride_k_c * esz + 15 * 16 >= (1LL << 32)) return PA_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(a->key_cache) | reinterpret_cast<uintptr_t>(a->value_cache) |
+       reinterpret_cast<uintptr_t>(a->query)) & 15)
+    return PA_ERR_BAD_SHAPE;
+
+  const int Ge = a->q_len * a->group_size;
+  const int nt = (Ge + 15) / 16;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  const bool pt = a->kv_quant_mode == PA_QUANT_PER_TOKEN;
+  if (a->kv_dtype == PA_DTYPE_FP8_E4M3FN)
+    return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true>(*a, nt, stream)
+              : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false>(*a, nt, stream);
+  if (pt) return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
+  return launch_partition_nt<PA_DTYPE_BF16, false>(*a, nt, stream);
+}
+
+int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!a->output) return PA_ERR_NULL_POINTER;
+  if (a->stride_out_h % 2 || a->stride_out_s % 2 || a->stride_tmp_g % 2 || a->stride_tmp_p % 2 ||
+      a->stride_tmp_h % 2 || a->stride_tmp_s % 2)
+    return PA_ERR_BAD_SHAPE;
+  const long long rows = (long long)a->num_seqs * a->num_kv_heads * a->q_len * a->group_size;
+  const long long blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  hipLaunchKernelGGL(pa_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return PA_OK;
+}
+
+int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
+  int rc = pa_decode_partition(a, hip_stream);
+  if (rc) return rc;
+  return pa_decode_reduce(a, hip_stream);
+}
+
+int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream) {
+  if (!codes || !out) return PA_ERR_NULL_POINTER;
+  if (n <= 0) return PA_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(pa_fp8_decode_kernel, dim3((n + 255) / 256), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(hip_stream), codes, out, n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return PA_OK;
+}
+
+}  // extern "C"
