@@ -1,0 +1,286 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (via the Python entry point or the
+raw ctypes functions), against the CPU oracle on the same seeded inputs.
+
+Tolerances.  End to end the bar is atol 2e-2 / rtol 2e-2 on the bf16 output (torch.allclose rule
+|a-b| <= atol + rtol*|b|).  Stage-wise: max_logits and exp_sums are f32 results of a bf16 x bf16
+MFMA dot product with f32 accumulation, compared at 1e-4 (+1e-5 relative); tmp_output carries
+the bf16 rounding of P and of the stored value, compared at 2e-2 like the output.
+"""
+import ctypes as C
+import math
+
+import pytest
+import torch
+
+from oracle import pa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+ATOL = RTOL = 2e-2
+
+
+def _ctx(*v):
+    return torch.tensor(v, dtype=torch.int32)
+
+
+def _run(wl, dev, *, partition_size=256, alibi=None, transposed=False, **kw):
+    import triton_op_amd as T
+
+    g = wl.to(dev)
+    out = torch.full_like(g.query, float("nan"))
+    res = T.paged_attention_decode(
+        out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale, g.q_len,
+        g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+        alibi_slopes=None if alibi is None else alibi.to(dev), partition_size=partition_size,
+        query_lens=g.q_lens, **kw)
+    torch.cuda.synchronize()
+    return out.cpu(), res
+
+
+def _oracle(wl, alibi=None, seq_ids=None):
+    return O.paged_attention_decode_oracle(
+        wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, alibi, seq_ids)
+
+
+def _check_stages(wl, res, partition_size, alibi=None):
+    P = res["maximum_logits"].shape[2]
+    ml, es, to = O.partition_stage(
+        wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, alibi, partition_size, P)
+    gml, ges = res["maximum_logits"].cpu(), res["exponential_sums"].cpu()
+    gto = res["temporary_output"].float().cpu()
+    fin = torch.isfinite(ml)
+    assert torch.equal(gml[~fin], ml[~fin]), "rows with no visible key must hold max=-inf"
+    torch.testing.assert_close(gml[fin], ml[fin], atol=1e-4, rtol=1e-5)
+    torch.testing.assert_close(ges, es, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(gto, to, atol=ATOL, rtol=RTOL)
+    # the reduce kernel alone, on the kernel's own partition buffers, against the closed-form merge
+    merged = O.reduce_stage(gml, ges, gto, wl.context_lens, partition_size)
+    return merged
+
+
+def _make(**kw):
+    from triton_op_amd import workloads as W
+
+    kw.setdefault("name", "t")
+    kw.setdefault("seed", 7)
+    return W.make_decode_workload(**kw)
+
+
+def test_fp8_dequant_table_on_device(cuda, pa_lib):
+    codes = torch.arange(256, dtype=torch.uint8, device=cuda)
+    out = torch.empty(256, dtype=torch.float32, device=cuda)
+    assert pa_lib.pa_debug_fp8_decode(codes.data_ptr(), out.data_ptr(), 256, None) == 0
+    torch.cuda.synchronize()
+    tab = torch.from_numpy(O.e4m3fn_table())
+    o = out.cpu()
+    assert torch.equal(torch.isnan(o), torch.isnan(tab))
+    ok = ~torch.isnan(tab)
+    assert torch.equal(o[ok], tab[ok])
+
+
+CASES = {
+    # the reference sweep's awkward shapes: groups 5/10 (non power of two), ctx 4097, qlen 1..4
+    "fp8_g8": dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000)),
+    "fp8_g8_boundaries": dict(batch=6, num_q_heads=8, num_kv_heads=1, context_lens=_ctx(1, 255, 256, 257, 512, 4097)),
+    "fp8_g5_q2": dict(batch=3, num_q_heads=5, num_kv_heads=1, context_lens=_ctx(257, 33, 700), q_len=2),
+    "fp8_g10_q3": dict(batch=2, num_q_heads=10, num_kv_heads=1, context_lens=_ctx(513, 100), q_len=3),
+    "fp8_g16_q4": dict(batch=2, num_q_heads=64, num_kv_heads=4, context_lens=_ctx(513, 4100), q_len=4),
+    "fp8_g16_q1": dict(batch=2, num_q_heads=16, num_kv_heads=1, context_lens=_ctx(4096, 17)),
+    "fp8_token_g16_q4": dict(batch=3, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(257, 33, 700), q_len=4,
+                             scale_mode="token"),
+    "fp8_token_g8_q1": dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(257, 33, 1700),
+                            scale_mode="token"),
+    "fp8_token_ragged": dict(batch=4, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(257, 33, 700, 5), q_len=4,
+                             q_lens=_ctx(1, 2, 3, 4), scale_mode="token"),
+    "bf16_g8": dict(batch=4, num_q_heads=8, num_kv_heads=1, context_lens=_ctx(1, 300, 1024, 77), kv_dtype="bf16",
+                    scale_mode="none"),
+    "bf16_g16_q2": dict(batch=2, num_q_heads=16, num_kv_heads=1, context_lens=_ctx(300, 77), kv_dtype="bf16",
+                        scale_mode="none", q_len=2),
+    "bf16_g16_q4": dict(batch=2, num_q_heads=16, num_kv_heads=1, context_lens=_ctx(600, 77), kv_dtype="bf16",
+                        scale_mode="none", q_len=4),
+    "fp8_bs1024_q2": dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(1500, 1024, 3000),
+                          block_size=1024, q_len=2),
+    "fp8_bs64": dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(1500, 63, 300), block_size=64),
+    "fp8_transV_bs16": dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000),
+                            transposed_v=True),
+    "fp8_transV_bs1024": dict(batch=2, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(1500, 3000),
+                              block_size=1024, transposed_v=True),
+    "bf16_transV_bs64": dict(batch=2, num_q_heads=8, num_kv_heads=2, context_lens=_ctx(150, 300), block_size=64,
+                             kv_dtype="bf16", scale_mode="none", transposed_v=True),
+}
+
+
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("partition_size", [256, 512])
+def test_parity_stagewise_and_end_to_end(cuda, name, partition_size):
+    wl = _make(**CASES[name])
+    print(f"case={name} partition_size={partition_size}", flush=True)
+    out, res = _run(wl, cuda, partition_size=partition_size)
+    ref = _oracle(wl)
+    assert not torch.isnan(out.float()).any()
+    torch.testing.assert_close(out.float(), ref.float(), atol=ATOL, rtol=RTOL)
+    merged = _check_stages(wl, res, partition_size)
+    torch.testing.assert_close(out.float(), merged.float(), atol=4e-3, rtol=8e-3)  # bf16 rounding only
+    thr = O.error_stats(out, ref)["max_diff_thr"]
+    assert thr < 1e-2, thr
+
+
+def test_alibi(cuda):
+    wl = _make(**CASES["fp8_g8"])
+    slopes = torch.linspace(0.01, 0.3, wl.num_q_heads, dtype=torch.float32)
+    out, res = _run(wl, cuda, alibi=slopes)
+    torch.testing.assert_close(out.float(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
+    _check_stages(wl, res, 256, slopes)
+
+
+def test_golden_fixtures(cuda):
+    import glob
+    import os
+
+    import triton_op_amd as T
+    from tests.golden.make_golden import load_case
+
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+    assert files
+    for f in files:
+        c = load_case(f)
+        d = {k: (v.to(cuda) if torch.is_tensor(v) else v) for k, v in c.items()}
+        out = torch.empty_like(d["query"])
+        T.paged_attention_decode(out, d["query"], d["key_cache"], d["value_cache"], d["context_lens"],
+                                 d["block_tables"], c["softmax_scale"], c["q_len"], int(c["context_lens"].max()),
+                                 torch.bfloat16, None, d["key_scale"], d["value_scale"])
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out.double().cpu(), c["expected"], atol=ATOL, rtol=RTOL)
+        err = float(((out.double().cpu() - c["expected"]).abs() / (1 + c["expected"].abs())).max())
+        assert err < 6e-3, (f, err)
+
+
+def test_stale_cache_contents_are_never_used(cuda):
+    """Slots past context_len in the last page, pages named by unused block-table entries, and their
+    per-token scales, hold NaN bytes: the result must not change (and must not be NaN)."""
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(5, 250, 1001), scale_mode="token", q_len=2)
+    ref_out, _ = _run(wl, cuda)
+    kc, vc = wl.key_cache.clone().view(torch.uint8), wl.value_cache.clone().view(torch.uint8)
+    ks, vs = wl.key_scale.clone(), wl.value_scale.clone()
+    used = set()
+    for b in range(3):
+        ctx = int(wl.context_lens[b])
+        for i in range((ctx + 15) // 16):
+            page = int(wl.block_tables[b, i])
+            used.add(page)
+            live = min(16, ctx - 16 * i)
+            kc[page, :, :, live:, :] = 0x7F
+            vc[page, :, :, live:] = 0x7F
+            ks[page, :, live:] = float("nan")
+            vs[page, :, live:] = float("nan")
+    spare = [p for p in range(kc.shape[0]) if p not in used]
+    for p in spare:
+        kc[p], vc[p], ks[p], vs[p] = 0x7F, 0x7F, float("nan"), float("nan")
+    bt = wl.block_tables.clone()
+    for b in range(3):
+        n = (int(wl.context_lens[b]) + 15) // 16
+        bt[b, n:] = spare[0]
+    wl2 = type(wl)(**{**wl.__dict__, "key_cache": kc.view(torch.float8_e4m3fn), "value_cache": vc.view(torch.float8_e4m3fn),
+                     "key_scale": ks, "value_scale": vs, "block_tables": bt})
+    out, _ = _run(wl2, cuda)
+    assert torch.equal(out.view(torch.int16), ref_out.view(torch.int16))
+
+
+def test_block_permutation_invariance_bit_exact(cuda):
+    wl = _make(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(700, 64, 2049, 300), q_len=2)
+    base, _ = _run(wl, cuda)
+    n = wl.key_cache.shape[0]
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(3))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(n)
+    wl2 = type(wl)(**{**wl.__dict__, "key_cache": wl.key_cache[perm], "value_cache": wl.value_cache[perm],
+                     "block_tables": inv[wl.block_tables.long()].to(torch.int32)})
+    out, _ = _run(wl2, cuda)
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+
+
+def test_caller_buffers_strided_inputs_and_twin_entry_point(cuda):
+    from triton_op_amd import pa_decode_triton
+
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000))
+    g = wl.to(cuda)
+    ref = _oracle(wl)
+    P, ge = 4, 8
+    es = torch.full((3, 2, P + 2, ge), 7.0, device=cuda)[:, :, :P]  # non-contiguous partition axis
+    ml = torch.full((3, 2, P + 2, ge), 7.0, device=cuda)[:, :, :P]
+    to = torch.full((3, 2, P, ge, 128), 7.0, dtype=torch.bfloat16, device=cuda)
+    qpad = torch.zeros(3, 16, 256, dtype=torch.bfloat16, device=cuda)
+    qpad[:, :, :128] = g.query
+    q = qpad[:, :, :128]  # row stride 256
+    out = torch.empty(3, 16, 128, dtype=torch.bfloat16, device=cuda)
+    res = pa_decode_triton.paged_attention_decode(out, q, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                                                  g.softmax_scale, g.max_context_len, torch.bfloat16, g.key_scale,
+                                                  g.value_scale, exp_sums=es, max_logits=ml, tmp_output=to)
+    torch.cuda.synchronize()
+    assert res["exp_sums"].data_ptr() == es.data_ptr() and res["partition_size"] == 256
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
+    # partitions a sequence does not reach are left untouched (sequence 1 has 64 tokens: 1 partition)
+    assert (es[1, :, 1:] == 7.0).all() and (to[1, :, 1:] == 7.0).all()
+
+
+def test_fp8_query_with_scales(cuda):
+    """FP8 query with a per-row scale, the reference Gluon entry point's own contract
+    (pa_decode_triton_gluon_fp8.py:747-755,889-903)."""
+    import triton_op_amd as T
+    from triton_op_amd import kv_layout as L
+
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000), q_len=2, scale_mode="token")
+    qq, qs = L.pertoken_quant(wl.query.float())
+    g = wl.to(cuda)
+    out = torch.empty_like(g.query)
+    T.paged_attention_decode(out, qq.to(cuda), g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, qs.to(cuda), g.key_scale,
+                             g.value_scale)
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode_oracle(qq, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                          wl.softmax_scale, 2, wl.key_scale, wl.value_scale, query_scale=qs)
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
+    qs0 = torch.tensor(float(wl.query.float().abs().max()) / 448.0)
+    qq0 = (wl.query.float() / qs0).to(torch.float8_e4m3fn)
+    T.paged_attention_decode(out, qq0.to(cuda), g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, qs0.to(cuda), g.key_scale,
+                             g.value_scale)
+    torch.cuda.synchronize()
+    ref0 = O.paged_attention_decode_oracle(qq0, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                           wl.softmax_scale, 2, wl.key_scale, wl.value_scale, query_scale=qs0)
+    torch.testing.assert_close(out.float().cpu(), ref0.float(), atol=ATOL, rtol=RTOL)
+
+
+def test_c_abi_rejects_bad_arguments(cuda, pa_lib):
+    import triton_op_amd as T
+    from triton_op_amd import _cabi
+
+    wl = _make(batch=2, num_q_heads=8, num_kv_heads=1, context_lens=_ctx(100, 300)).to(cuda)
+    out = torch.empty_like(wl.query)
+    plan = T.plan_decode(out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                         wl.softmax_scale, 1, 300, torch.bfloat16, None, wl.key_scale, wl.value_scale)
+    a = plan.args
+    assert pa_lib.pa_decode(None, None) == -1
+    for field, bad, code in (("struct_size", 8, -2), ("head_size", 64, -3), ("block_size", 32, -3),
+                             ("partition_size", 100, -4), ("key_cache", None, -1), ("num_seqs", 0, -4),
+                             ("stride_k_b", 8, -4)):
+        good = getattr(a, field)
+        setattr(a, field, bad)
+        assert pa_lib.pa_decode(C.byref(a), None) == code, field
+        setattr(a, field, good)
+    assert pa_lib.pa_decode(C.byref(a), C.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    assert pa_lib.pa_decode_error_string(-3).decode().startswith("unsupported")
+
+
+@pytest.mark.parametrize("name,batch,ctx_scale", [
+    ("c1", None, 1.0), ("c2", 8, 0.25), ("c3", 6, 0.125), ("c4", 1, 1 / 32), ("c5", 12, 0.25)])
+def test_scaled_down_benchmark_configs(cuda, name, batch, ctx_scale):
+    from triton_op_amd import workloads as W
+
+    wl = W.make_config(name, batch=batch, ctx_scale=ctx_scale)
+    print(f"config={wl.name} ctx={wl.context_lens.tolist()}", flush=True)
+    out, res = _run(wl, cuda, partition_size=None)
+    torch.testing.assert_close(out.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)

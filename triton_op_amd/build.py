@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
-    "-std=c++17",
+    "-std=c++20",
     "-fno-strict-aliasing",
     "-fPIC",
     "-shared",

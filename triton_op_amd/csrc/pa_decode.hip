@@ -27,6 +27,10 @@
 
 #include "../../include/pa_decode.h"
 
+#ifndef PA_CVT_SCALEF32
+#define PA_CVT_SCALEF32 0
+#endif
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -48,12 +52,22 @@ union Bf16x8Bits {
   u32x4 u;
 };
 
-// two FP8 e4m3fn bytes -> two f32 (v_cvt_pk_f32_fp8), then keep the upper 16 bits of each:
-// exact, since an e4m3 value has 3 mantissa bits and bf16 keeps 7.
+// two FP8 e4m3fn bytes -> two bf16, exactly (an e4m3 value has 3 mantissa bits, bf16 keeps 7)
 __device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t word, bool high_half) {
+#if PA_CVT_SCALEF32
+  union {
+    bf16x2 v;
+    uint32_t u;
+  } r;
+  r.v = high_half ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)word, 1.0f, true)
+                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)word, 1.0f, false);
+  return r.u;
+#else
+  // v_cvt_pk_f32_fp8, then keep the upper 16 bits of each f32
   f32x2 f = high_half ? __builtin_amdgcn_cvt_pk_f32_fp8((int)word, true)
                       : __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
   return __builtin_amdgcn_perm(__float_as_uint(f[1]), __float_as_uint(f[0]), 0x07060302u);
+#endif
 }
 
 __device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t lo, uint32_t hi) {
@@ -81,6 +95,33 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 
+// wave-uniform 32-bit load through the scalar (constant) path: no VGPR, no vmcnt slot
+__device__ __forceinline__ int sload_i32(const int* p) {
+  return *reinterpret_cast<const __attribute__((address_space(4))) int*>(reinterpret_cast<uintptr_t>(p));
+}
+__device__ __forceinline__ float sload_f32(const float* p) {
+  return *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(p));
+}
+
+// max / sum over the four lanes {l, l^16, l^32, l^48}: v_permlane{16,32}_swap exchange 16- and
+// 32-lane halves inside the VALU (no LDS round trip)
+__device__ __forceinline__ float quad_row_max(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  u = __float_as_uint(x);
+  auto b = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_row_sum(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  u = __float_as_uint(x);
+  auto b = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // keep the first `n` (0..16) bytes of a 16-byte vector, zero the rest
 __device__ __forceinline__ u32x4 keep_first_bytes(u32x4 v, int n) {
 #pragma unroll
@@ -103,74 +144,16 @@ struct StepData {
   f32x4 vs[PER_TOKEN ? 4 : 1];
 };
 
-struct WaveCtx {
-  const char* kbase;   // key_cache + head offset (bytes)
-  const char* vbase;   // value_cache + head offset (bytes)
-  const float* ksbase; // key_scale + head offset
-  const float* vsbase;
-  int64_t k_block_bytes, v_block_bytes, kvs_block;
-  uint32_t k_lane_off[4];  // per-lane byte offset of K load ld inside a tile
-  uint32_t v_row_bytes;    // byte distance between consecutive head dims of V
-  uint32_t v_half_bytes;   // byte distance between the two 8-token halves of a bf16 V tile
-  int log2_bs;
-  int bs_mask;
-  int v_transposed;
-  int64_t v_group_bytes;   // transposed V: bytes between consecutive 16-token tiles of a page
-};
-
-// page id of the 16-token tile `tile` (uniform value broadcast from the page-id register)
-__device__ __forceinline__ int tile_page(const int* pages4, int step_in_chunk, int j) {
-  return __builtin_amdgcn_readlane(pages4[step_in_chunk], 16 * j);
-}
-
-template <int KVT, bool PER_TOKEN>
-__device__ __forceinline__ void load_step(StepData<KVT, PER_TOKEN>& sd, const WaveCtx& c, int page_lane,
-                                          int tok0, int first_tile_tok, int last_tile_tok, int li, int kg,
-                                          int esz) {
-  // K: tile j of the step, same page for the whole wave
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    int t = tok0 + 16 * j;
-    t = t > last_tile_tok ? last_tile_tok : t;
-    int page = __builtin_amdgcn_readlane(page_lane, 16 * j);
-    const char* tb = c.kbase + (int64_t)page * c.k_block_bytes + (int64_t)(t & c.bs_mask) * 16;
-#pragma unroll
-    for (int ld = 0; ld < StepData<KVT, PER_TOKEN>::NKL; ++ld) sd.k[j][ld] = load16(tb + c.k_lane_off[ld]);
-    if constexpr (PER_TOKEN) {
-      const float* sb = c.ksbase + (int64_t)page * c.kvs_block + (t & c.bs_mask) + 4 * kg;
-      sd.ks[j] = *reinterpret_cast<const f32x4*>(sb);
-      const float* vb = c.vsbase + (int64_t)page * c.kvs_block + (t & c.bs_mask) + 4 * kg;
-      sd.vs[j] = *reinterpret_cast<const f32x4*>(vb);
-    }
-  }
-  // V: lane group kg owns tile kg of the step
-  {
-    int t = tok0 + 16 * kg;
-    t = t > last_tile_tok ? last_tile_tok : t;
-    int off = t & c.bs_mask;
-    const char* tb = c.vbase + (int64_t)page_lane * c.v_block_bytes +
-                     (c.v_transposed ? (int64_t)(off >> 4) * c.v_group_bytes : (int64_t)off * esz);
-#pragma unroll
-    for (int db = 0; db < 8; ++db) {
-      const char* rp = tb + (uint32_t)(16 * db + li) * c.v_row_bytes;
-#pragma unroll
-      for (int hf = 0; hf < StepData<KVT, PER_TOKEN>::NVL; ++hf) sd.v[db][hf] = load16(rp + hf * c.v_half_bytes);
-    }
-  }
-  (void)first_tile_tok;
-}
-
-template <int NT>
-struct RowState {
-  float m[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
-  float l[NT];      // this lane's share of the running sum of exp2(s - m)
-  f32x4 acc[NT][8]; // O^T: [16*db + 4*kg + r][row]
-};
-
-// DEPTH 2 keeps the next step's loads in flight during the current step's arithmetic (two register
-// copies of a step's cache data); DEPTH 1 loads and computes in turn and leaves the overlap to the
-// other waves of the SIMD.  OCC is the number of waves per SIMD the register budget is cut for.
-template <int NT, int KVT, bool PER_TOKEN, int WAVES, int DEPTH, int OCC>
+// The partition kernel.  OCC is the number of waves per SIMD the register budget is cut for.
+//
+// Software pipeline of one wave (each line is issued in order; loads return in order):
+//   QK(s)      needs K(s)            -> then K(s+1) is loaded into the registers K(s) just left
+//   softmax(s)                          (K(s+1) and V(s) in flight)
+//   PV(s)      needs V(s)            -> then V(s+1) is loaded into the registers V(s) just left
+// so about one step (16 KiB) of cache data per wave is in flight at any time without a second
+// register copy.  Steps that need no masking and have a successor run in a branch-free loop, so
+// the compiler's vmcnt waits stay partial; the last step(s) go through the masked variants.
+template <int NT, int KVT, bool PER_TOKEN, int WAVES, int OCC>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_kernel(const PaDecodeArgs a) {
   constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
@@ -180,11 +163,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   __shared__ __attribute__((aligned(16))) char p_lds[WAVES][NT][16 * kPRowBytes];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15;
   const int kg = lane >> 4;
 
-  // ---- which (sequence, head, partition) -------------------------------------------------
+  // ---- which (sequence, head, partition): all wave-uniform -----------------------------------------
   const int P = a.max_num_partitions;
   const int Hkv = a.num_kv_heads;
   const long long wid = (long long)blockIdx.x * WAVES + wave;
@@ -194,16 +177,94 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int part = (int)((wid / Hkv) % P);
   const int b = (int)(wid / ((long long)Hkv * P));
 
-  const int ctx = a.context_lens[b];
+  const int ctx = sload_i32(a.context_lens + b);
   const int part_start = part * a.partition_size;
   if (part_start >= ctx) return;
   const int part_end = min(part_start + a.partition_size, ctx);
   const int G = a.group_size;
   const int Ge = a.q_len * G;  // rows per kv head in the buffers
-  const int qb = a.q_lens ? a.q_lens[b] : a.q_len;
+  const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
   const int rows_valid = qb * G;
 
-  // ---- per-lane row bookkeeping -----------------------------------------------------------
+  // ---- cache addressing -------------------------------------------------------------------------------
+  const int log2_bs = 31 - __builtin_clz(a.block_size);
+  const int bs_mask = a.block_size - 1;
+  const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h * esz;
+  const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h * esz;
+  const int64_t k_block_bytes = a.stride_k_b * esz;
+  const int64_t v_block_bytes = a.stride_v_b * esz;
+  const float* ksbase = PER_TOKEN ? a.key_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  const float* vsbase = PER_TOKEN ? a.value_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  uint32_t k_lane_off[SD::NKL];  // per-lane byte offset of K load ld inside a tile
+#pragma unroll
+  for (int ld = 0; ld < SD::NKL; ++ld) k_lane_off[ld] = (uint32_t)((4 * ld + kg) * a.stride_k_c * esz + li * 16);
+  // V: byte offset of this lane's head dim inside a tile, distance of the second 8-token half
+  // (bf16 only) and, for the transposed layout, of consecutive 16-token tiles of a page
+  const uint32_t v_row_bytes = a.v_transposed ? 16u : (uint32_t)(a.stride_v_2 * esz);
+  const uint32_t v_half_bytes = a.v_transposed ? (uint32_t)(a.stride_v_2 * esz) : 16u;
+  const int64_t v_tile_bytes = a.v_transposed ? a.stride_v_2 * esz * esz : 16 * esz;
+  uint32_t v_lane_off[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) v_lane_off[db] = (uint32_t)(16 * db + li) * v_row_bytes;
+
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const int last_tile_tok = (part_end - 1) & ~15;  // first token of the last tile that holds a live token
+
+  // page ids of the four tiles of the step that starts at token tok0 (scalar loads; tiles past the
+  // last live one repeat it, so no block-table slot or page beyond the sequence is ever touched)
+  struct Pages {
+    int p[4];
+    int off[4];  // token offset of the tile inside its page
+  };
+  auto load_pages = [&](int tok0) {
+    Pages pg;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int t = tok0 + 16 * j;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      pg.p[j] = sload_i32(bt + (t >> log2_bs));
+      pg.off[j] = t & bs_mask;
+    }
+    return pg;
+  };
+  auto issue_k = [&](SD& sd, const Pages& pg) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const char* tb = kbase + (int64_t)pg.p[j] * k_block_bytes + (int64_t)pg.off[j] * 16;
+#pragma unroll
+      for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16(tb + k_lane_off[ld]);
+      if constexpr (PER_TOKEN) {
+        const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + pg.off[j] + 4 * kg;
+        sd.ks[j] = *reinterpret_cast<const f32x4*>(ksbase + so);
+      }
+    }
+  };
+  auto issue_v = [&](SD& sd, const Pages& pg) {
+    // lane group kg owns tile kg of the step
+    const int page = kg == 0 ? pg.p[0] : (kg == 1 ? pg.p[1] : (kg == 2 ? pg.p[2] : pg.p[3]));
+    const int off = kg == 0 ? pg.off[0] : (kg == 1 ? pg.off[1] : (kg == 2 ? pg.off[2] : pg.off[3]));
+    const char* tb = vbase + (int64_t)page * v_block_bytes + (int64_t)(off >> 4) * v_tile_bytes;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < SD::NVL; ++hf) sd.v[db][hf] = load16(tb + v_lane_off[db] + hf * v_half_bytes);
+    }
+    if constexpr (PER_TOKEN) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + pg.off[j] + 4 * kg;
+        sd.vs[j] = *reinterpret_cast<const f32x4*>(vsbase + so);
+      }
+    }
+  };
+
+  // ---- first loads go out before anything else is set up ---------------------------------------------
+  SD sd;
+  Pages pg_cur = load_pages(part_start);
+  issue_k(sd, pg_cur);
+  issue_v(sd, pg_cur);
+
+  // ---- per-lane row bookkeeping -------------------------------------------------------------------------
   int limit[NT];      // number of visible keys of this lane's query row
   float slope2[NT];   // ALiBi slope * log2e
   const bool has_alibi = a.alibi_slopes != nullptr;
@@ -212,104 +273,72 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     int row = 16 * nt + li;
     int t = row / G;
     limit[nt] = row < rows_valid ? ctx - (qb - 1 - t) : 0;
-    slope2[nt] = (has_alibi && row < rows_valid) ? a.alibi_slopes[h * G + (row - t * G)] * kLog2e : 0.f;
+    slope2[nt] = 0.f;
+    if (has_alibi && row < rows_valid) slope2[nt] = a.alibi_slopes[h * G + (row - t * G)] * kLog2e;
   }
   const int min_limit = ctx - (qb - 1);  // keys below this index are visible to every real row
 
-  // ---- query: B operand of S^T = K Q^T ------------------------------------------------------
+  // ---- query: B operand of S^T = K Q^T --------------------------------------------------------------------
   // k-step s of a tile covers, for lane group kg, the 8 head dims the K load puts in that slot.
+  // Rows past the last real one are loaded from row 0 and zeroed, which keeps this branch-free.
   bf16x8 qreg[NT][4];
   {
-    const char* qb_ptr = (const char*)a.query;
+    const char* q_ptr = (const char*)a.query;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      int row = 16 * nt + li;
-      bool ok = row < rows_valid;
+      const int row = 16 * nt + li;
+      const bool ok = row < rows_valid;
+      const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (ok ? row : 0)) * a.stride_q_h;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
+        const int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
         Bf16x8Bits q;
-        q.u = u32x4{0, 0, 0, 0};
-        if (ok) {
-          int64_t e = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + row) * a.stride_q_h + dim;
-          if (a.query_dtype == PA_DTYPE_BF16) {
-            q.u = load16(qb_ptr + e * 2);
-          } else {
-            u32x2 raw = *reinterpret_cast<const u32x2*>(qb_ptr + e);
-            q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
-          }
+        if (a.query_dtype == PA_DTYPE_BF16) {
+          q.u = load16(q_ptr + (e0 + dim) * 2);
+        } else {
+          u32x2 raw = *reinterpret_cast<const u32x2*>(q_ptr + e0 + dim);
+          q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
         }
+        if (!ok) q.u = u32x4{0, 0, 0, 0};
         qreg[nt][s] = q.v;
       }
     }
   }
   // per-row query scale (FP8 query) multiplies the logits of that row
-  float qscale[NT];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    int row = 16 * nt + li;
-    qscale[nt] = 1.f;
-    if (a.query_quant_mode == PA_QUANT_PER_TENSOR) qscale[nt] = a.query_scale[0];
-    if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row < rows_valid)
-      qscale[nt] = a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
-  }
-
-  // ---- cache addressing ---------------------------------------------------------------------
-  WaveCtx c;
-  c.log2_bs = 31 - __builtin_clz(a.block_size);
-  c.bs_mask = a.block_size - 1;
-  c.kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h * esz;
-  c.vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h * esz;
-  c.k_block_bytes = a.stride_k_b * esz;
-  c.v_block_bytes = a.stride_v_b * esz;
-  c.kvs_block = a.stride_kvscale_b;
-  c.ksbase = PER_TOKEN ? a.key_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
-  c.vsbase = PER_TOKEN ? a.value_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
-#pragma unroll
-  for (int ld = 0; ld < 4; ++ld) c.k_lane_off[ld] = (uint32_t)((4 * ld + kg) * a.stride_k_c * esz + li * 16);
-  c.v_transposed = a.v_transposed;
-  if (a.v_transposed) {
-    c.v_row_bytes = 16;
-    c.v_group_bytes = a.stride_v_2 * esz * esz;  // a 16-token tile is 16/x = esz groups of x tokens
-    c.v_half_bytes = (uint32_t)(a.stride_v_2 * esz);
-  } else {
-    c.v_row_bytes = (uint32_t)(a.stride_v_2 * esz);
-    c.v_group_bytes = 0;
-    c.v_half_bytes = 16;
-  }
   float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
   if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
-    k_tensor_scale = a.key_scale[0];
-    v_tensor_scale = a.value_scale[0];
+    k_tensor_scale = sload_f32(a.key_scale);
+    v_tensor_scale = sload_f32(a.value_scale);
   }
   const float scale2 = a.softmax_scale * k_tensor_scale * kLog2e;
-
-  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
-  const int last_tile_tok = (part_end - 1) & ~15;  // first token of the last tile that holds a live token
-
-  // page ids: lane group kg keeps the page of tile (4*step + kg) for the 4 steps of a 256-token chunk
-  auto load_pages = [&](int chunk_tok0, int* pages4) {
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      int t = chunk_tok0 + kStepTokens * s + 16 * kg;
-      t = t > last_tile_tok ? last_tile_tok : t;
-      pages4[s] = bt[t >> c.log2_bs];
-    }
-  };
-
-  RowState<NT> st;
+  float rscale[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    st.m[nt] = -INFINITY;
-    st.l[nt] = 0.f;
+    const int row = 16 * nt + li;
+    float qs = 1.f;
+    if (a.query_quant_mode == PA_QUANT_PER_TENSOR) qs = sload_f32(a.query_scale);
+    if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row < rows_valid)
+      qs = a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
+    rscale[nt] = scale2 * qs;
+  }
+
+  float m_run[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
+  float l_run[NT];      // this lane's share of the running sum of exp2(s - m)
+  f32x4 acc[NT][8];     // O^T: acc[nt][db][r] is head dim 16*db + 4*kg + r of query row 16*nt + li
 #pragma unroll
-    for (int db = 0; db < 8; ++db) st.acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int nt = 0; nt < NT; ++nt) {
+    m_run[nt] = -INFINITY;
+    l_run[nt] = 0.f;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
   char* plds = &p_lds[wave][0][0];
 
-  // ---- one step of 64 tokens -------------------------------------------------------------------
-  auto compute_step = [&](SD& sd, int tok0) {
+  // ---- one step of 64 tokens ------------------------------------------------------------------------------
+  // FULL: every token of the step is visible to every row and there is no ALiBi term.
+  // PREFETCH: a next step exists; its K and V are requested as soon as this step's are consumed.
+  auto step = [&]<bool FULL, bool PREFETCH>(int tok0, const Pages& pg_next) {
     // S^T tiles
     f32x4 s[NT][4];
 #pragma unroll
@@ -335,35 +364,27 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         }
       }
     }
-
-    const bool full = (tok0 + kStepTokens <= min_limit) && !has_alibi;  // wave-uniform
-    if (!full) {
-      // zero the V bytes of tokens at or beyond ctx (stale cache contents may decode to NaN)
-      int nvalid = ctx - (tok0 + 16 * kg);
-      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+    f32x4 ks_cur[PER_TOKEN ? 4 : 1];
+    if constexpr (PER_TOKEN) {
 #pragma unroll
-      for (int db = 0; db < 8; ++db) {
-        if constexpr (kFp8) {
-          sd.v[db][0] = keep_first_bytes(sd.v[db][0], nvalid);
-        } else {
-          sd.v[db][0] = keep_first_bytes(sd.v[db][0], 2 * (nvalid > 8 ? 8 : nvalid));
-          sd.v[db][1] = keep_first_bytes(sd.v[db][1], 2 * (nvalid > 8 ? nvalid - 8 : 0));
-        }
-      }
+      for (int j = 0; j < 4; ++j) ks_cur[j] = sd.ks[j];
     }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREFETCH) issue_k(sd, pg_next);
+    __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const float rs = scale2 * qscale[nt];
+      const float rs = rscale[nt];
       float mx = -INFINITY;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float v = s[nt][j][r] * rs;
-          if constexpr (PER_TOKEN) v *= sd.ks[j][r];
-          if (!full) {
-            int col = tok0 + 16 * j + 4 * kg + r;
+          if constexpr (PER_TOKEN) v *= ks_cur[j][r];
+          if constexpr (!FULL) {
+            const int col = tok0 + 16 * j + 4 * kg + r;
             v += slope2[nt] * (float)(col - ctx + 1);
             v = col < limit[nt] ? v : -INFINITY;
           }
@@ -371,12 +392,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
           mx = fmaxf(mx, v);
         }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(st.m[nt], mx);
+      mx = quad_row_max(mx);
+      const float m_new = fmaxf(m_run[nt], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = fast_exp2(st.m[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
-      st.m[nt] = m_new;
+      const float alpha = fast_exp2(m_run[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
+      m_run[nt] = m_new;
       float psum = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -388,7 +408,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         if constexpr (PER_TOKEN) {
           // a masked token's scale may be stale memory (NaN): its weight must stay exactly 0
           f32x4 vsc = sd.vs[j];
-          if (!full) {
+          if constexpr (!FULL) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) vsc[r] = s[nt][j][r] == -INFINITY ? 0.f : vsc[r];
           }
@@ -402,9 +422,24 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         pk[1] = pack_bf16x2(p2, p3);
         *reinterpret_cast<u32x2*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes + (16 * j + 4 * kg) * 2) = pk;
       }
-      st.l[nt] = st.l[nt] * alpha + psum;
+      l_run[nt] = l_run[nt] * alpha + psum;
 #pragma unroll
-      for (int db = 0; db < 8; ++db) st.acc[nt][db] *= alpha;
+      for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha;
+    }
+
+    if constexpr (!FULL) {
+      // zero the V bytes of tokens at or beyond ctx (stale cache contents may decode to NaN)
+      int nvalid = ctx - (tok0 + 16 * kg);
+      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        if constexpr (kFp8) {
+          sd.v[db][0] = keep_first_bytes(sd.v[db][0], nvalid);
+        } else {
+          sd.v[db][0] = keep_first_bytes(sd.v[db][0], 2 * (nvalid > 8 ? 8 : nvalid));
+          sd.v[db][1] = keep_first_bytes(sd.v[db][1], 2 * (nvalid > 8 ? nvalid - 8 : 0));
+        }
+      }
     }
 
     // the P tile is written and read by this wave only; LDS operations of one wave complete in order
@@ -435,47 +470,41 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-          st.acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nt], st.acc[nt][db], 0, 0, 0);
+          acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nt], acc[nt][db], 0, 0, 0);
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREFETCH) issue_v(sd, pg_next);
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   };
 
-  // ---- main loop: chunks of 256 tokens, 4 steps each, next step's data in flight -------------------
+  // ---- main loop ----------------------------------------------------------------------------------------------
   const int n_steps = (part_end - part_start + kStepTokens - 1) / kStepTokens;
-  int pages_cur[4], pages_next[4];
-  load_pages(part_start, pages_cur);
-  SD buf0, buf1;
-  load_step<KVT, PER_TOKEN>(buf0, c, pages_cur[0], part_start, part_start, last_tile_tok, li, kg, esz);
-
-  int step = 0;
-  for (int chunk_tok0 = part_start; chunk_tok0 < part_end; chunk_tok0 += kChunkTokens) {
-    const bool more_chunks = chunk_tok0 + kChunkTokens < part_end;
-    if (more_chunks) load_pages(chunk_tok0 + kChunkTokens, pages_next);
-#pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4) {
-      const int tok0 = chunk_tok0 + kStepTokens * s4;
-      if (step < n_steps) {  // wave-uniform
-        const bool has_next = step + 1 < n_steps;
-        const int np = s4 < 3 ? pages_cur[s4 + 1] : pages_next[0];
-        if constexpr (DEPTH == 2) {
-          SD& cur = (s4 & 1) ? buf1 : buf0;
-          SD& nxt = (s4 & 1) ? buf0 : buf1;
-          if (has_next)
-            load_step<KVT, PER_TOKEN>(nxt, c, np, tok0 + kStepTokens, part_start, last_tile_tok, li, kg, esz);
-          compute_step(cur, tok0);
-        } else {
-          compute_step(buf0, tok0);
-          if (has_next)
-            load_step<KVT, PER_TOKEN>(buf0, c, np, tok0 + kStepTokens, part_start, last_tile_tok, li, kg, esz);
-        }
-      }
-      ++step;
-    }
-#pragma unroll
-    for (int s = 0; s < 4; ++s) pages_cur[s] = pages_next[s];
+  // leading steps that need no masking: tok0 + 64 <= min_limit
+  int n_full = has_alibi ? 0 : (min_limit - part_start) / kStepTokens;
+  n_full = n_full < 0 ? 0 : n_full;
+  const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
+  int sidx = 0;
+  int tok0 = part_start;
+  Pages pg_next = load_pages(part_start + kStepTokens);
+  for (; sidx < n_fast; ++sidx) {
+    Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
+    step.template operator()<true, true>(tok0, pg_next);
+    pg_next = pg_after;
+    tok0 += kStepTokens;
   }
+  for (; sidx < n_steps - 1; ++sidx) {
+    Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
+    step.template operator()<false, true>(tok0, pg_next);
+    pg_next = pg_after;
+    tok0 += kStepTokens;
+  }
+  if (n_full >= n_steps)
+    step.template operator()<true, false>(tok0, pg_next);
+  else
+    step.template operator()<false, false>(tok0, pg_next);
 
   // ---- epilogue: normalise, store m (natural-log domain), l and the bf16 partial output -----------
   const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
@@ -483,11 +512,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
                                      (int64_t)part * a.stride_tmp_p) * 2;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    float l = st.l[nt];
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
+    float l = quad_row_sum(l_run[nt]);
     const int row = 16 * nt + li;
-    float m_out = st.m[nt] * (1.0f / kLog2e);
+    float m_out = m_run[nt] * (1.0f / kLog2e);
     if (row >= rows_valid) {  // padding rows of a ragged batch: no visible key
       l = 0.f;
       m_out = -INFINITY;
@@ -501,7 +528,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       char* rp = tmp + (int64_t)row * a.stride_tmp_g * 2;
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
-        f32x4 o = st.acc[nt][db] * inv;
+        f32x4 o = acc[nt][db] * inv;
         u32x2 pk;
         pk[0] = pack_bf16x2(o[0], o[1]);
         pk[1] = pack_bf16x2(o[2], o[3]);
@@ -612,13 +639,11 @@ int check_common(const PaDecodeArgs* a) {
 template <int NT, int KVT, bool PT>
 int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   constexpr int W = 1;
-  constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
-  constexpr int DEPTH = (NT == 1 && kFp8) ? 2 : 1;
   constexpr int OCC = NT == 1 ? 2 : 1;
   long long total = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
   long long blocks = (total + W - 1) / W;
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, W, DEPTH, OCC>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
+  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, W, OCC>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
