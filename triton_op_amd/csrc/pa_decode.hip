@@ -539,22 +539,24 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// reduce: one wave per output row, two head dims per lane; streams over the partitions
+// reduce: one wave per output row, two head dims per lane.  Lane p of a 64-partition chunk owns
+// (m_p, l_p); the weights w_p = l_p e^{m_p - M} are broadcast with v_readlane while the partial
+// outputs of the chunk stream in, eight loads in flight per lane.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
   const int lane = threadIdx.x & 63;
   const int Ge = a.q_len * a.group_size;
-  const long long rid = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long long rid = (long long)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const long long total = (long long)a.num_seqs * a.num_kv_heads * Ge;
   if (rid >= total) return;
   const int row = (int)(rid % Ge);
   const int h = (int)((rid / Ge) % a.num_kv_heads);
   const int b = (int)(rid / ((long long)Ge * a.num_kv_heads));
 
-  const int ctx = a.context_lens[b];
+  const int ctx = sload_i32(a.context_lens + b);
   int n = (ctx + a.partition_size - 1) / a.partition_size;
   n = n > a.max_num_partitions ? a.max_num_partitions : n;
-  const int qb = a.q_lens ? a.q_lens[b] : a.q_len;
+  const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
 
   uint32_t* out = reinterpret_cast<uint32_t*>((char*)a.output +
                                               ((int64_t)b * a.stride_out_s + (int64_t)(h * Ge + row) * a.stride_out_h) * 2) + lane;
@@ -569,42 +571,49 @@ __global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
                     ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h + (int64_t)row * a.stride_tmp_g) * 2 +
                     lane * 4;
   const int64_t tp = a.stride_tmp_p * 2;
+  const int64_t sp = a.stride_es_p;
 
-  // global max over partitions
-  float M = -INFINITY;
-  for (int p = lane; p < n; p += 64) M = fmaxf(M, ml[(int64_t)p * a.stride_es_p]);
+  // this lane's (m, l) of the first chunk, and the global max
+  float m0 = lane < n ? ml[(int64_t)lane * sp] : -INFINITY;
+  float l0 = lane < n ? es[(int64_t)lane * sp] : 0.f;
+  float M = m0;
+  for (int p = lane + 64; p < n; p += 64) M = fmaxf(M, ml[p * sp]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
   const float M_safe = M == -INFINITY ? 0.f : M;
 
   float acc0 = 0.f, acc1 = 0.f, wsum = 0.f;
-  int p = 0;
-  for (; p + 4 <= n; p += 4) {
-    float w[4];
-    uint32_t t[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float m = ml[(int64_t)(p + u) * a.stride_es_p];
-      float l = es[(int64_t)(p + u) * a.stride_es_p];
-      w[u] = l > 0.f ? l * __expf(m - M_safe) : 0.f;
-      t[u] = *reinterpret_cast<const uint32_t*>(tmp + (int64_t)(p + u) * tp);
+  for (int c0 = 0; c0 < n; c0 += 64) {
+    const int cnt = n - c0 < 64 ? n - c0 : 64;
+    float m = m0, l = l0;
+    if (c0) {
+      m = lane < cnt ? ml[(int64_t)(c0 + lane) * sp] : -INFINITY;
+      l = lane < cnt ? es[(int64_t)(c0 + lane) * sp] : 0.f;
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      wsum += w[u];
-      acc0 += bf16_bits_to_f32(t[u] & 0xffffu) * w[u];
-      acc1 += bf16_bits_to_f32(t[u] >> 16) * w[u];
-    }
-  }
-  for (; p < n; ++p) {
-    float m = ml[(int64_t)p * a.stride_es_p];
-    float l = es[(int64_t)p * a.stride_es_p];
-    float w = l > 0.f ? l * __expf(m - M_safe) : 0.f;
-    uint32_t t = *reinterpret_cast<const uint32_t*>(tmp + (int64_t)p * tp);
+    const float w = l > 0.f ? l * __expf(m - M_safe) : 0.f;
     wsum += w;
-    acc0 += bf16_bits_to_f32(t & 0xffffu) * w;
-    acc1 += bf16_bits_to_f32(t >> 16) * w;
+    const char* tc = tmp + (int64_t)c0 * tp;
+    int u = 0;
+    for (; u + 8 <= cnt; u += 8) {
+      uint32_t t[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) t[i] = *reinterpret_cast<const uint32_t*>(tc + (int64_t)(u + i) * tp);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float wi = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w), u + i));
+        acc0 += bf16_bits_to_f32(t[i] & 0xffffu) * wi;
+        acc1 += __uint_as_float(t[i] & 0xffff0000u) * wi;
+      }
+    }
+    for (; u < cnt; ++u) {
+      const uint32_t t = *reinterpret_cast<const uint32_t*>(tc + (int64_t)u * tp);
+      const float wi = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w), u));
+      acc0 += bf16_bits_to_f32(t & 0xffffu) * wi;
+      acc1 += __uint_as_float(t & 0xffff0000u) * wi;
+    }
   }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) wsum += __shfl_xor(wsum, o);
   const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
   *out = pack_bf16x2(acc0 * inv, acc1 * inv);
 }
