@@ -24,6 +24,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/pa_decode.h"
 
@@ -39,6 +40,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
 
 constexpr int kHeadSize = 128;
 constexpr int kStepTokens = 64;     // tokens per pipeline step (4 tiles of 16)
@@ -122,6 +124,19 @@ __device__ __forceinline__ float quad_row_sum(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// 4x4 transpose over (lane group l>>4, register): afterwards register k of lane group g holds what
+// register g of lane group k held
+__device__ __forceinline__ void quad_transpose(uint32_t (&d)[4]) {
+  auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+  auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+  auto s01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+  auto s23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+  d[0] = s01[0];
+  d[1] = s01[1];
+  d[2] = s23[0];
+  d[3] = s23[1];
+}
+
 // keep the first `n` (0..16) bytes of a 16-byte vector, zero the rest
 __device__ __forceinline__ u32x4 keep_first_bytes(u32x4 v, int n) {
 #pragma unroll
@@ -153,14 +168,23 @@ struct StepData {
 // so about one step (16 KiB) of cache data per wave is in flight at any time without a second
 // register copy.  Steps that need no masking and have a successor run in a branch-free loop, so
 // the compiler's vmcnt waits stay partial; the last step(s) go through the masked variants.
-template <int NT, int KVT, bool PER_TOKEN, int WAVES, int OCC>
+//
+// BS16 (block size 16) turns every stride inside a page into a compile-time constant, so the loads
+// of a tile share one address register pair and differ by immediate offsets.
+// FP8MATH (FP8 cache only) feeds the cache bytes to the FP8 MFMAs as they are: Q and P are split into
+// an FP8 head and an FP8 residual (q*c = hi + lo, each product exact in the f32 accumulator), which
+// keeps them at bf16-like precision, costs two MFMAs where the bf16 path has one, and removes every
+// FP8->bf16 conversion and the LDS round trip of P (a 4x4 lane-group transpose with
+// v_permlane{16,32}_swap puts P into the B-operand layout).
+template <int NT, int KVT, bool PER_TOKEN, bool FP8MATH, bool BS16, int WAVES, int OCC, int DEPTH>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_kernel(const PaDecodeArgs a) {
   constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
+  static_assert(kFp8 || !FP8MATH, "FP8 MFMA path needs an FP8 cache");
   constexpr int esz = kFp8 ? 1 : 2;
   typedef StepData<KVT, PER_TOKEN> SD;
 
-  __shared__ __attribute__((aligned(16))) char p_lds[WAVES][NT][16 * kPRowBytes];
+  __shared__ __attribute__((aligned(16))) char p_lds[FP8MATH ? 1 : WAVES][FP8MATH ? 1 : NT][FP8MATH ? 16 : 16 * kPRowBytes];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -195,17 +219,21 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int64_t v_block_bytes = a.stride_v_b * esz;
   const float* ksbase = PER_TOKEN ? a.key_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
   const float* vsbase = PER_TOKEN ? a.value_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  const uint32_t k_chunk_bytes = BS16 ? 256u : (uint32_t)(a.stride_k_c * esz);
   uint32_t k_lane_off[SD::NKL];  // per-lane byte offset of K load ld inside a tile
 #pragma unroll
-  for (int ld = 0; ld < SD::NKL; ++ld) k_lane_off[ld] = (uint32_t)((4 * ld + kg) * a.stride_k_c * esz + li * 16);
+  for (int ld = 0; ld < SD::NKL; ++ld) k_lane_off[ld] = (uint32_t)(kg * k_chunk_bytes + li * 16) + 4 * ld * k_chunk_bytes;
   // V: byte offset of this lane's head dim inside a tile, distance of the second 8-token half
   // (bf16 only) and, for the transposed layout, of consecutive 16-token tiles of a page
-  const uint32_t v_row_bytes = a.v_transposed ? 16u : (uint32_t)(a.stride_v_2 * esz);
-  const uint32_t v_half_bytes = a.v_transposed ? (uint32_t)(a.stride_v_2 * esz) : 16u;
-  const int64_t v_tile_bytes = a.v_transposed ? a.stride_v_2 * esz * esz : 16 * esz;
+  // (with block size 16 the plain and the transposed FP8 layouts are the same bytes; for bf16 they
+  // differ, so the constant-stride form is used for the plain layout only)
+  const bool vt = a.v_transposed;
+  const uint32_t v_row_bytes = BS16 ? 16u * esz : (vt ? 16u : (uint32_t)(a.stride_v_2 * esz));
+  const uint32_t v_half_bytes = BS16 ? 16u : (vt ? (uint32_t)(a.stride_v_2 * esz) : 16u);
+  const int64_t v_tile_bytes = BS16 ? 16 * esz : (vt ? a.stride_v_2 * esz * esz : 16 * esz);
   uint32_t v_lane_off[8];
 #pragma unroll
-  for (int db = 0; db < 8; ++db) v_lane_off[db] = (uint32_t)(16 * db + li) * v_row_bytes;
+  for (int db = 0; db < 8; ++db) v_lane_off[db] = li * v_row_bytes + 16 * db * v_row_bytes;
 
   const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
   const int last_tile_tok = (part_end - 1) & ~15;  // first token of the last tile that holds a live token
@@ -259,10 +287,20 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   };
 
   // ---- first loads go out before anything else is set up ---------------------------------------------
-  SD sd;
-  Pages pg_cur = load_pages(part_start);
-  issue_k(sd, pg_cur);
-  issue_v(sd, pg_cur);
+  const int n_steps = (part_end - part_start + kStepTokens - 1) / kStepTokens;
+  // DEPTH 2: steps alternate between two buffers, each refilled in place for the step after next;
+  // DEPTH 1: one buffer, refilled in place for the next step
+  SD buf_a, buf_b;
+  {
+    Pages pg0 = load_pages(part_start);
+    issue_k(buf_a, pg0);
+    issue_v(buf_a, pg0);
+    if (DEPTH == 2 && n_steps > 1) {
+      Pages pg1 = load_pages(part_start + kStepTokens);
+      issue_k(buf_b, pg1);
+      issue_v(buf_b, pg1);
+    }
+  }
 
   // ---- per-lane row bookkeeping -------------------------------------------------------------------------
   int limit[NT];      // number of visible keys of this lane's query row
@@ -321,6 +359,44 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       qs = a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
     rscale[nt] = scale2 * qs;
   }
+  // FP8 math: q * cq = hi + lo with hi, lo in e4m3 (|q * cq| <= 224); the logits are divided by cq again
+  i32x8 qhi[FP8MATH ? NT : 1], qlo[FP8MATH ? NT : 1];
+  if constexpr (FP8MATH) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      float f[32];
+      float amax = 0.f;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        Bf16x8Bits q;
+        q.v = qreg[nt][s4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          f[8 * s4 + 2 * e] = bf16_bits_to_f32(q.u[e] & 0xffffu);
+          f[8 * s4 + 2 * e + 1] = __uint_as_float(q.u[e] & 0xffff0000u);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(f[e]));
+      amax = quad_row_max(amax);
+      const float cq = amax > 0.f ? 224.f / amax : 1.f;
+      rscale[nt] *= amax > 0.f ? amax * (1.f / 224.f) : 1.f;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        const float x0 = f[4 * w] * cq, x1 = f[4 * w + 1] * cq, x2 = f[4 * w + 2] * cq, x3 = f[4 * w + 3] * cq;
+        int hi = 0, lo = 0;
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, hi, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(x2, x3, hi, true);
+        const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+        const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(x0 - b01[0], x1 - b01[1], lo, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(x2 - b23[0], x3 - b23[1], lo, true);
+        qhi[nt][w] = hi;
+        qlo[nt][w] = lo;
+      }
+    }
+  }
+  float v_run = 1e-30f;  // FP8 math with per-token V scales: running max of the scales seen so far
 
   float m_run[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
   float l_run[NT];      // this lane's share of the running sum of exp2(s - m)
@@ -338,13 +414,22 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // ---- one step of 64 tokens ------------------------------------------------------------------------------
   // FULL: every token of the step is visible to every row and there is no ALiBi term.
   // PREFETCH: a next step exists; its K and V are requested as soon as this step's are consumed.
-  auto step = [&]<bool FULL, bool PREFETCH>(int tok0, const Pages& pg_next) {
+  auto step = [&]<bool FULL, bool PREFETCH>(SD& sd, int tok0, const Pages& pg_next) {
     // S^T tiles
     f32x4 s[NT][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) s[nt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (FP8MATH) {
+        const i32x8 ka = {(int)sd.k[j][0][0], (int)sd.k[j][0][1], (int)sd.k[j][0][2], (int)sd.k[j][0][3],
+                          (int)sd.k[j][1][0], (int)sd.k[j][1][1], (int)sd.k[j][1][2], (int)sd.k[j][1][3]};
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          s[nt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi[nt], s[nt][j], 0, 0, 0, 0, 0, 0);
+          s[nt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo[nt], s[nt][j], 0, 0, 0, 0, 0, 0);
+        }
+      } else
 #pragma unroll
       for (int ld = 0; ld < SD::NKL; ++ld) {
         if constexpr (kFp8) {
@@ -372,6 +457,32 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (PREFETCH) issue_k(sd, pg_next);
     __builtin_amdgcn_sched_barrier(0);
+
+    // FP8 math, per-token V scales: P carries v_scale / v_run (<= 1); the accumulator is kept in units
+    // of the running maximum v_run
+    float vfac = 1.f, pmul = 256.f;
+    f32x4 vs_cur[(PER_TOKEN && FP8MATH) ? 4 : 1];
+    if constexpr (PER_TOKEN && FP8MATH) {
+      float vmx = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vs_cur[j] = sd.vs[j];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (!FULL) {
+            const int col = tok0 + 16 * j + 4 * kg + r;
+            vs_cur[j][r] = col < ctx ? vs_cur[j][r] : 0.f;
+          }
+          vmx = fmaxf(vmx, vs_cur[j][r]);
+        }
+      }
+      vmx = quad_row_max(vmx);
+      const float v_new = fmaxf(v_run, vmx);
+      vfac = v_run / v_new;
+      pmul = 256.f / v_new;
+      v_run = v_new;
+    }
+    uint32_t ph[FP8MATH ? NT : 1][4], pl[FP8MATH ? NT : 1][4];  // FP8 math: P head / residual, 4 tokens per dword
 
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -405,6 +516,28 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         float p2 = fast_exp2(s[nt][j][2] - m_safe);
         float p3 = fast_exp2(s[nt][j][3] - m_safe);
         psum += (p0 + p1) + (p2 + p3);
+        if constexpr (FP8MATH) {
+          if constexpr (PER_TOKEN) {
+            p0 *= vs_cur[j][0];
+            p1 *= vs_cur[j][1];
+            p2 *= vs_cur[j][2];
+            p3 *= vs_cur[j][3];
+          }
+          p0 *= pmul;
+          p1 *= pmul;
+          p2 *= pmul;
+          p3 *= pmul;
+          int hi = 0, lo = 0;
+          hi = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, hi, false);
+          hi = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, hi, true);
+          const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+          const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+          lo = __builtin_amdgcn_cvt_pk_fp8_f32(p0 - b01[0], p1 - b01[1], lo, false);
+          lo = __builtin_amdgcn_cvt_pk_fp8_f32(p2 - b23[0], p3 - b23[1], lo, true);
+          ph[nt][j] = (uint32_t)hi;
+          pl[nt][j] = (uint32_t)lo;
+          continue;
+        }
         if constexpr (PER_TOKEN) {
           // a masked token's scale may be stale memory (NaN): its weight must stay exactly 0
           f32x4 vsc = sd.vs[j];
@@ -423,8 +556,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         *reinterpret_cast<u32x2*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes + (16 * j + 4 * kg) * 2) = pk;
       }
       l_run[nt] = l_run[nt] * alpha + psum;
+      const float alpha_acc = alpha * vfac;
 #pragma unroll
-      for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha;
+      for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha_acc;
     }
 
     if constexpr (!FULL) {
@@ -440,6 +574,34 @@ void pa_partition_kernel(const PaDecodeArgs a) {
           sd.v[db][1] = keep_first_bytes(sd.v[db][1], 2 * (nvalid > 8 ? nvalid - 8 : 0));
         }
       }
+    }
+
+    if constexpr (FP8MATH) {
+      // lane group kg holds, per tile j, tokens 4kg..4kg+3; the B operand of O^T += V^T P^T wants lane
+      // group kg to hold all 16 tokens of tile kg: a 4x4 transpose over (lane group, register)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        quad_transpose(ph[nt]);
+        quad_transpose(pl[nt]);
+      }
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int db = 0; db < 8; ++db) {
+          const long va = (long)(((uint64_t)sd.v[db][0][2 * hf + 1] << 32) | sd.v[db][0][2 * hf]);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const long bh = (long)(((uint64_t)ph[nt][2 * hf + 1] << 32) | ph[nt][2 * hf]);
+            const long bl = (long)(((uint64_t)pl[nt][2 * hf + 1] << 32) | pl[nt][2 * hf]);
+            acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(va, bh, acc[nt][db], 0, 0, 0);
+            acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(va, bl, acc[nt][db], 0, 0, 0);
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PREFETCH) issue_v(sd, pg_next);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
     }
 
     // the P tile is written and read by this wave only; LDS operations of one wave complete in order
@@ -480,31 +642,65 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     __builtin_amdgcn_wave_barrier();
   };
 
-  // ---- main loop ----------------------------------------------------------------------------------------------
-  const int n_steps = (part_end - part_start + kStepTokens - 1) / kStepTokens;
+  // ---- main loop -------------------------------------------------------------------------------------------
   // leading steps that need no masking: tok0 + 64 <= min_limit
   int n_full = has_alibi ? 0 : (min_limit - part_start) / kStepTokens;
   n_full = n_full < 0 ? 0 : n_full;
-  const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
   int sidx = 0;
   int tok0 = part_start;
-  Pages pg_next = load_pages(part_start + kStepTokens);
-  for (; sidx < n_fast; ++sidx) {
-    Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
-    step.template operator()<true, true>(tok0, pg_next);
-    pg_next = pg_after;
-    tok0 += kStepTokens;
+  if constexpr (DEPTH == 2) {
+    // pairs of unmasked steps that both have a step two ahead to request
+    const int n_pf = n_steps - 2;
+    const int n_fast = (n_full < n_pf ? n_full : n_pf) & ~1;
+    Pages pg_a = load_pages(part_start + 2 * kStepTokens);  // pages of the step buf_a is refilled for
+    Pages pg_b = load_pages(part_start + 3 * kStepTokens);
+    for (; sidx < n_fast; sidx += 2) {
+      const Pages na = load_pages(tok0 + 4 * kStepTokens);
+      step.template operator()<true, true>(buf_a, tok0, pg_a);
+      const Pages nb = load_pages(tok0 + 5 * kStepTokens);
+      step.template operator()<true, true>(buf_b, tok0 + kStepTokens, pg_b);
+      pg_a = na;
+      pg_b = nb;
+      tok0 += 2 * kStepTokens;
+    }
+    // the two steps already requested, then (ALiBi, or an odd step left over) load-and-compute
+    if (n_full >= n_steps) {
+      step.template operator()<true, false>(buf_a, tok0, pg_a);
+      if (sidx + 1 < n_steps) step.template operator()<true, false>(buf_b, tok0 + kStepTokens, pg_b);
+      sidx += 2;
+    } else {
+      step.template operator()<false, false>(buf_a, tok0, pg_a);
+      if (sidx + 1 < n_steps) step.template operator()<false, false>(buf_b, tok0 + kStepTokens, pg_b);
+      sidx += 2;
+      tok0 += 2 * kStepTokens;
+      for (; sidx < n_steps; ++sidx) {
+        const Pages pg = load_pages(tok0);
+        issue_k(buf_a, pg);
+        issue_v(buf_a, pg);
+        step.template operator()<false, false>(buf_a, tok0, pg);
+        tok0 += kStepTokens;
+      }
+    }
+  } else {
+    const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
+    Pages pg_next = load_pages(part_start + kStepTokens);
+    for (; sidx < n_fast; ++sidx) {
+      const Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
+      step.template operator()<true, true>(buf_a, tok0, pg_next);
+      pg_next = pg_after;
+      tok0 += kStepTokens;
+    }
+    for (; sidx < n_steps - 1; ++sidx) {
+      const Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
+      step.template operator()<false, true>(buf_a, tok0, pg_next);
+      pg_next = pg_after;
+      tok0 += kStepTokens;
+    }
+    if (n_full >= n_steps)
+      step.template operator()<true, false>(buf_a, tok0, pg_next);
+    else
+      step.template operator()<false, false>(buf_a, tok0, pg_next);
   }
-  for (; sidx < n_steps - 1; ++sidx) {
-    Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
-    step.template operator()<false, true>(tok0, pg_next);
-    pg_next = pg_after;
-    tok0 += kStepTokens;
-  }
-  if (n_full >= n_steps)
-    step.template operator()<true, false>(tok0, pg_next);
-  else
-    step.template operator()<false, false>(tok0, pg_next);
 
   // ---- epilogue: normalise, store m (natural-log domain), l and the bf16 partial output -----------
   const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
@@ -519,7 +715,8 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       l = 0.f;
       m_out = -INFINITY;
     }
-    const float inv = l > 0.f ? v_tensor_scale / l : 0.f;
+    float inv = l > 0.f ? v_tensor_scale / l : 0.f;
+    if constexpr (FP8MATH) inv *= (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f);
     if (row < Ge) {
       if (kg == 0) {
         a.max_logits[es_off + row] = m_out;
@@ -645,14 +842,15 @@ int check_common(const PaDecodeArgs* a) {
   return PA_OK;
 }
 
-template <int NT, int KVT, bool PT>
+template <int NT, int KVT, bool PT, bool FP8MATH, bool BS16>
 int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   constexpr int W = 1;
   constexpr int OCC = NT == 1 ? 2 : 1;
+  constexpr int DEPTH = (NT == 1 && FP8MATH && !PT) ? 2 : 1;
   long long total = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
   long long blocks = (total + W - 1) / W;
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, W, OCC>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
+  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, FP8MATH, BS16, W, OCC, DEPTH>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
@@ -661,13 +859,13 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   return PA_OK;
 }
 
-template <int KVT, bool PT>
+template <int KVT, bool PT, bool FP8MATH, bool BS16>
 int launch_partition_nt(const PaDecodeArgs& a, int nt, hipStream_t stream) {
   switch (nt) {
-    case 1: return launch_partition_w<1, KVT, PT>(a, stream);
-    case 2: return launch_partition_w<2, KVT, PT>(a, stream);
+    case 1: return launch_partition_w<1, KVT, PT, FP8MATH, BS16>(a, stream);
+    case 2: return launch_partition_w<2, KVT, PT, FP8MATH, BS16>(a, stream);
     case 3:
-    case 4: return launch_partition_w<4, KVT, PT>(a, stream);
+    case 4: return launch_partition_w<4, KVT, PT, FP8MATH, BS16>(a, stream);
   }
   return PA_ERR_UNSUPPORTED;
 }
@@ -748,11 +946,18 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
   const int nt = (Ge + 15) / 16;
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   const bool pt = a->kv_quant_mode == PA_QUANT_PER_TOKEN;
-  if (a->kv_dtype == PA_DTYPE_FP8_E4M3FN)
-    return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true>(*a, nt, stream)
-              : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false>(*a, nt, stream);
+  if (a->kv_dtype == PA_DTYPE_FP8_E4M3FN) {
+    // constant in-page strides: block size 16 with the default dense layout
+    const bool bs16 = a->block_size == 16 && a->stride_k_c == 256 &&
+                      (a->v_transposed ? a->stride_v_2 == 2048 : a->stride_v_2 == 16);
+    if (bs16)
+      return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true, true>(*a, nt, stream)
+                : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true, true>(*a, nt, stream);
+    return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true, false>(*a, nt, stream)
+              : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true, false>(*a, nt, stream);
+  }
   if (pt) return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
-  return launch_partition_nt<PA_DTYPE_BF16, false>(*a, nt, stream);
+  return launch_partition_nt<PA_DTYPE_BF16, false, false, false>(*a, nt, stream);
 }
 
 int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
