@@ -2,9 +2,12 @@
 raw ctypes functions), against the CPU oracle on the same seeded inputs.
 
 Tolerances.  End to end the bar is atol 2e-2 / rtol 2e-2 on the bf16 output (torch.allclose rule
-|a-b| <= atol + rtol*|b|).  Stage-wise: max_logits and exp_sums are f32 results of a bf16 x bf16
-MFMA dot product with f32 accumulation, compared at 1e-4 (+1e-5 relative); tmp_output carries
-the bf16 rounding of P and of the stored value, compared at 2e-2 like the output.
+|a-b| <= atol + rtol*|b|).  Stage-wise: with an FP8 cache the kernel multiplies the cache bytes on the
+FP8 MFMAs and carries the bf16 query as an FP8 head plus an FP8 residual (about 2^-8 relative per
+element, like bf16 itself), so a scaled logit differs from the f32 oracle by a few 1e-3: max_logits
+is compared at atol 4e-3 + rtol 2e-3 and exp_sums at rtol 1e-2; with a bf16 cache (bf16 MFMA, exact
+products) both are compared at 1e-4.  tmp_output carries the rounding of P and of the stored bf16
+value and is compared at 2e-2 like the output.
 """
 import ctypes as C
 import math
@@ -52,8 +55,12 @@ def _check_stages(wl, res, partition_size, alibi=None):
     gto = res["temporary_output"].float().cpu()
     fin = torch.isfinite(ml)
     assert torch.equal(gml[~fin], ml[~fin]), "rows with no visible key must hold max=-inf"
-    torch.testing.assert_close(gml[fin], ml[fin], atol=1e-4, rtol=1e-5)
-    torch.testing.assert_close(ges, es, atol=1e-4, rtol=1e-4)
+    if wl.key_cache.dtype == torch.bfloat16:
+        torch.testing.assert_close(gml[fin], ml[fin], atol=1e-4, rtol=1e-5)
+        torch.testing.assert_close(ges, es, atol=1e-4, rtol=1e-4)
+    else:
+        torch.testing.assert_close(gml[fin], ml[fin], atol=4e-3, rtol=2e-3)
+        torch.testing.assert_close(ges, es, atol=1e-3, rtol=1e-2)
     torch.testing.assert_close(gto, to, atol=ATOL, rtol=RTOL)
     # the reduce kernel alone, on the kernel's own partition buffers, against the closed-form merge
     merged = O.reduce_stage(gml, ges, gto, wl.context_lens, partition_size)
@@ -113,11 +120,12 @@ CASES = {
 
 
 @pytest.mark.parametrize("name", list(CASES))
-@pytest.mark.parametrize("partition_size", [256, 512])
+@pytest.mark.parametrize("partition_size", [256, 512, 1024, 4096])
 def test_parity_stagewise_and_end_to_end(cuda, name, partition_size):
     wl = _make(**CASES[name])
     print(f"case={name} partition_size={partition_size}", flush=True)
     out, res = _run(wl, cuda, partition_size=partition_size)
+    assert res["partition_size"] == partition_size
     ref = _oracle(wl)
     assert not torch.isnan(out.float()).any()
     torch.testing.assert_close(out.float(), ref.float(), atol=ATOL, rtol=RTOL)

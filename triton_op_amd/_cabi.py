@@ -57,12 +57,14 @@ _lib = None
 _lock = threading.Lock()
 
 
-def load_library(path: str = LIB_PATH) -> C.CDLL:
-    """dlopen the HIP library and check that its struct layout matches this binding."""
+def load_library(path: str = None) -> C.CDLL:
+    """dlopen the HIP library and check that its struct layout matches this binding.
+    The environment variable PA_DECODE_LIB names another build of the library to load instead."""
     global _lib
     with _lock:
         if _lib is not None:
             return _lib
+        path = path or os.environ.get("PA_DECODE_LIB") or LIB_PATH
         if not os.path.exists(path):
             raise PaDecodeLibraryError(
                 f"{path} is missing: build it with `python -m triton_op_amd.build` "
