@@ -1,0 +1,157 @@
+"""CPU-side tests: the C-ABI library loads and exports every symbol the header declares, the ctypes
+struct matches it, the host-side argument checks raise the reference's errors, the tuning layer's
+choices, and the workload generators."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from triton_op_amd import _cabi, kv_layout as L, workloads as W
+import triton_op_amd as T
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header():
+    with open(os.path.join(ROOT, "include", "pa_decode.h")) as f:
+        return f.read()
+
+
+def test_library_exports_every_declared_symbol(pa_lib):
+    text = re.sub(r"/\*.*?\*/", "", _header(), flags=re.S)
+    declared = set(re.findall(r"\b(pa_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(_cabi.EXPORTED_SYMBOLS), declared ^ set(_cabi.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(pa_lib, name), name
+
+
+def test_struct_layout_and_version(pa_lib):
+    assert pa_lib.pa_decode_abi_version() == _cabi.PA_DECODE_ABI_VERSION
+    assert pa_lib.pa_decode_args_size() == C.sizeof(_cabi.PaDecodeArgs)
+    # every field of the header's struct, in order
+    body = re.search(r"typedef struct PaDecodeArgs \{(.*?)\} PaDecodeArgs;", _header(), re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        names += [n.strip().lstrip("*") for n in re.sub(r"^(const\s+)?[a-z0-9_]+\s*\**", "", decl, count=1).split(",")]
+    assert names == [f[0] for f in _cabi.PaDecodeArgs._fields_]
+
+
+def test_error_strings_and_null_arguments(pa_lib):
+    assert pa_lib.pa_decode_error_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert pa_lib.pa_decode_error_string(code) not in (b"ok", b"unknown error code")
+    assert pa_lib.pa_decode(None, None) == -1
+    a = _cabi.PaDecodeArgs()
+    assert pa_lib.pa_decode_partition(C.byref(a), None) == -2  # struct_size not set
+    a.struct_size = C.sizeof(_cabi.PaDecodeArgs)
+    assert pa_lib.pa_decode_partition(C.byref(a), None) == -1  # buffers are NULL
+    assert pa_lib.pa_debug_fp8_decode(None, None, 4, None) == -1
+
+
+def test_partition_size_choices():
+    f = T.select_partition_size
+    # (num_seqs, kv heads, rows per group, longest context, block size, CUs)
+    assert f(64, 8, 8, 4096, 16, 256) == 4096      # c2: one partition, four waves per workgroup, no reduce
+    assert f(4, 8, 8, 131072, 16, 256) == 8192     # c4: 16 partitions x 32 (sequence, head) pairs x 4 waves
+    assert f(128, 8, 16, 32768, 1024, 256) == 8192  # c3
+    assert f(256, 8, 64, 65536, 16, 256) == 2048   # c5: 64 rows -> one wave per workgroup, <= 2048 tokens
+    assert f(4, 1, 8, 1024, 16, 256) == 256        # c1: tiny, the finest split
+    for args in [(1, 1, 1, 1, 16, 256), (3, 5, 7, 100000, 64, 304), (1000, 8, 16, 300, 16, 64)]:
+        ps = f(*args)
+        assert ps >= 256 and ps % 256 == 0
+    with pytest.raises(_cabi.PaDecodeLibraryError):
+        f(0, 8, 8, 4096, 16, 256)
+
+
+def _cpu_args(**over):
+    wl = W.make_decode_workload(name="v", seed=1, batch=2, num_q_heads=8, num_kv_heads=2,
+                                context_lens=torch.tensor([40, 300], dtype=torch.int32))
+    kw = dict(output=torch.empty_like(wl.query), query=wl.query, key_cache=wl.key_cache, value_cache=wl.value_cache,
+              sequence_lengths=wl.context_lens, block_tables=wl.block_tables, softmax_scale=wl.softmax_scale,
+              query_sequence_length=1, max_sequence_length=300, compute_type=torch.bfloat16, query_scale=None,
+              key_scale=wl.key_scale, value_scale=wl.value_scale)
+    kw.update(over)
+    return kw
+
+
+@pytest.mark.parametrize("over,msg", [
+    (dict(output=torch.empty(2, 8, 128)), "output tensor only support dtype"),
+    (dict(query=torch.empty(16, 128, dtype=torch.bfloat16)), "Expected 3D query tensor"),
+    (dict(key_cache=torch.empty(4, 2, 16, 128, dtype=torch.float8_e4m3fn)), "Expected 5D key_cache"),
+    (dict(value_cache=torch.empty(4, 2, 128, dtype=torch.float8_e4m3fn)), "Unsupported value cache shape"),
+    (dict(query_sequence_length=3), "is not num_kv_heads"),
+    (dict(key_scale=torch.ones(4, 2, 16), value_scale=torch.ones(4, 2, 16)), "Expected 4D key_scale"),
+    (dict(key_scale=torch.ones((), dtype=torch.float64)), "key_scale tensor only support dtype"),
+    (dict(key_scale=torch.ones(4, 2, 16, 1)), "same shape"),
+    (dict(value_scale=None), "given together"),
+    (dict(compute_type=torch.float16), "compute_type"),
+    (dict(sequence_lengths=torch.tensor([40, 300])), "int32"),
+    (dict(), "GPU only"),
+])
+def test_entry_point_rejects_bad_arguments(over, msg):
+    with pytest.raises(ValueError, match=msg):
+        T.plan_decode(**_cpu_args(**over))
+
+
+def test_entry_point_rejects_group_and_block_size():
+    wl = W.make_decode_workload(name="v", seed=1, batch=1, num_q_heads=80, num_kv_heads=1,
+                                context_lens=torch.tensor([40], dtype=torch.int32))
+    with pytest.raises(ValueError, match="exceeds maximum of 64"):
+        T.plan_decode(torch.empty_like(wl.query), wl.query, wl.key_cache, wl.value_cache, wl.context_lens,
+                      wl.block_tables, 0.1, 1, 40, torch.bfloat16, None, wl.key_scale, wl.value_scale)
+    kc = torch.empty(4, 1, 8, 32, 16, dtype=torch.float8_e4m3fn)
+    vc = torch.empty(4, 1, 128, 32, dtype=torch.float8_e4m3fn)
+    q = torch.empty(1, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="not in"):
+        T.plan_decode(torch.empty_like(q), q, kc, vc, torch.tensor([40], dtype=torch.int32),
+                      torch.zeros(1, 4, dtype=torch.int32), 0.1, 1, 40)
+
+
+def test_library_path_must_exist(monkeypatch):
+    monkeypatch.setattr(_cabi, "_lib", None)
+    with pytest.raises(_cabi.PaDecodeLibraryError, match="is missing"):
+        _cabi.load_library("/nonexistent/libpa_decode.so")
+    monkeypatch.undo()
+    assert _cabi.load_library() is not None
+
+
+def test_workload_generators_shapes_and_bytes():
+    wl = W.make_config("c1")
+    assert wl.query.shape == (4, 8, 128) and wl.key_cache.shape == (256, 1, 16, 16, 8)
+    assert wl.value_cache.shape == (256, 1, 128, 16) and wl.block_tables.shape == (4, 64)
+    assert sorted(wl.block_tables.flatten().tolist()) == list(range(256))  # a permutation of the pool
+    assert 1 <= int(wl.context_lens.min()) and int(wl.context_lens.max()) <= 1024
+    c2 = W.make_config("c2", batch=2, ctx_scale=0.125)
+    assert c2.key_cache.dtype == torch.float8_e4m3fn and c2.key_cache.shape[1:] == (8, 8, 16, 16)
+    assert c2.key_scale.dim() == 0 and c2.meta["pool_blocks"] == 80  # 1.25 x 2 x 512 / 16
+    assert c2.kv_bytes() == 2 * 512 * 8 * 128 * 2
+    assert len(set(c2.block_tables.flatten().tolist())) == c2.block_tables.numel()
+    c5 = W.make_config("c5", batch=6, ctx_scale=0.05)
+    assert c5.key_scale.shape == (c5.key_cache.shape[0], 8, 16, 1) and c5.q_lens is not None
+    assert c5.query.shape == (6, 8 * 4 * 16, 128)
+    assert c5.kv_bytes() == int(c5.context_lens.sum()) * 8 * (256 + 8)
+    # same seed, same tensors
+    again = W.make_config("c2", batch=2, ctx_scale=0.125)
+    assert torch.equal(again.key_cache.view(torch.uint8), c2.key_cache.view(torch.uint8))
+    assert torch.equal(again.block_tables, c2.block_tables)
+
+
+def test_per_token_quantised_cache_layout():
+    g = torch.Generator().manual_seed(3)
+    kc, vc = L.create_kv_cache(5, 16, 2, 128, torch.bfloat16, generator=g)
+    kq, ks, vq, vs = L.quantize_kv_cache_per_token(kc, vc)
+    assert kq.shape == (5, 2, 8, 16, 16) and vq.shape == (5, 2, 128, 16) and ks.shape == vs.shape == (5, 2, 16, 1)
+    ktok = L.key_cache_to_tokens(kc).float()  # [blocks, bs, Hkv, D]
+    back = L.key_cache_to_tokens(kq).float() * ks.permute(0, 2, 1, 3)
+    assert float((back - ktok).abs().max()) <= float(ktok.abs().max()) * 2.0 ** -4
+    vtok = L.value_cache_to_tokens(vc).float()
+    vback = L.value_cache_to_tokens(vq).float() * vs.permute(0, 2, 1, 3)
+    assert float((vback - vtok).abs().max()) <= float(vtok.abs().max()) * 2.0 ** -4
+    kq2, ks2, vq2, vs2 = L.quantize_kv_cache_per_tensor(kc, vc)
+    assert kq2.shape == kq.shape and ks2.dim() == 0
