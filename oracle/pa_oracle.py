@@ -217,11 +217,12 @@ def mha_extend(
     return out
 
 
-def _row_qlens(batch: int, qlen: Union[int, torch.Tensor, Sequence[int]]):
+def _row_qlens(batch: int, qlen: Union[int, torch.Tensor, Sequence[int]], q_max: Optional[int] = None):
+    """per-sequence query lengths and the number of query positions the packed rows are laid out for"""
     if isinstance(qlen, int):
-        return [qlen] * batch, qlen
+        return [qlen] * batch, (q_max or qlen)
     ql = [int(v) for v in qlen]
-    return ql, max(ql)
+    return ql, (q_max or max(ql))
 
 
 def paged_attention_decode_oracle(
@@ -237,6 +238,7 @@ def paged_attention_decode_oracle(
     alibi_slopes: Optional[torch.Tensor] = None,
     seq_ids: Optional[Sequence[int]] = None,
     query_scale: Optional[torch.Tensor] = None,
+    q_max: Optional[int] = None,
 ) -> torch.Tensor:
     """The oracle behind the entry point's own conventions: output [B, Hkv*qmax*G, D] in
     query's 16-bit dtype (bf16 when the query is FP8).  Rows of padded query positions
@@ -245,7 +247,7 @@ def paged_attention_decode_oracle(
     hkv = key_cache.shape[1]
     d = query.shape[-1]
     bs = key_cache.shape[-2]
-    qls, qmax = _row_qlens(batch, query_sequence_length)
+    qls, qmax = _row_qlens(batch, query_sequence_length, q_max)
     g = query.shape[1] // (hkv * qmax)
     out_dtype = query.dtype if query.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
     qf = query.to(torch.float32)
@@ -284,6 +286,7 @@ def partition_stage(
     partition_size: int = 256,
     max_num_partitions: Optional[int] = None,
     seq_ids: Optional[Sequence[int]] = None,
+    q_max: Optional[int] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(max_logits, exp_sums, tmp_output): [B,Hkv,P,Ge] f32 x2 and [B,Hkv,P,Ge,D] f32.
 
@@ -297,7 +300,7 @@ def partition_stage(
     hkv = key_cache.shape[1]
     d = query.shape[-1]
     bs = key_cache.shape[-2]
-    qls, qmax = _row_qlens(batch, query_sequence_length)
+    qls, qmax = _row_qlens(batch, query_sequence_length, q_max)
     g = query.shape[1] // (hkv * qmax)
     ge = qmax * g
     if max_num_partitions is None:
