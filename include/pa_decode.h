@@ -21,7 +21,12 @@
 extern "C" {
 #endif
 
-#define PA_DECODE_ABI_VERSION 1
+#define PA_DECODE_ABI_VERSION 2
+/* Size of the optional device workspace.  It holds a work-item counter: with it, ragged batches are launched
+ * as a resident grid that pulls live (sequence, partition, row tile, head) items from the counter instead
+ * of one workgroup per possible item.  It must be zero before the first call; every call leaves it zero.
+ * Calls that may overlap on the GPU need a workspace each. */
+#define PA_DECODE_WORKSPACE_BYTES 64
 
 /* element types */
 enum { PA_DTYPE_BF16 = 0, PA_DTYPE_FP8_E4M3FN = 1 };
@@ -78,6 +83,7 @@ typedef struct PaDecodeArgs {
   float* exp_sums;
   float* max_logits;
   void* tmp_output;
+  int32_t* workspace;         /* optional, >= PA_DECODE_WORKSPACE_BYTES, zero on entry; left zero on return */
 
   int32_t num_seqs;
   int32_t num_kv_heads;

@@ -12,7 +12,8 @@ import threading
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
-PA_DECODE_ABI_VERSION = 1
+PA_DECODE_ABI_VERSION = 2
+PA_DECODE_WORKSPACE_BYTES = 64
 PA_DTYPE_BF16, PA_DTYPE_FP8_E4M3FN = 0, 1
 PA_QUANT_NONE, PA_QUANT_PER_TENSOR, PA_QUANT_PER_TOKEN = -1, 0, 1
 
@@ -34,7 +35,8 @@ class PaDecodeArgs(C.Structure):
         [("struct_size", C.c_uint32), ("reserved0", C.c_int32)]
         + [(n, C.c_void_p) for n in (
             "output", "query", "key_cache", "value_cache", "context_lens", "block_tables", "q_lens",
-            "query_scale", "key_scale", "value_scale", "alibi_slopes", "exp_sums", "max_logits", "tmp_output")]
+            "query_scale", "key_scale", "value_scale", "alibi_slopes", "exp_sums", "max_logits", "tmp_output",
+            "workspace")]
         + [(n, C.c_int32) for n in (
             "num_seqs", "num_kv_heads", "group_size", "q_len", "head_size", "block_size",
             "max_num_partitions", "partition_size", "query_dtype", "kv_dtype", "query_quant_mode",

@@ -208,7 +208,9 @@ struct StepData {
 // keeps them at bf16-like precision, costs two MFMAs where the bf16 path has one, and removes every
 // FP8->bf16 conversion and the LDS round trip of P (a 4x4 lane-group transpose with
 // v_permlane{16,32}_swap puts P into the B-operand layout).
-template <int NT, int KVT, bool PER_TOKEN, bool FP8MATH, bool BS16, int WAVES, int OCC, int DEPTH>
+constexpr int kQueueMaxSeqs = 2048;  // sequences the item table of the queued launch can hold
+
+template <int NT, int KVT, bool PER_TOKEN, bool FP8MATH, bool BS16, int WAVES, int OCC, int DEPTH, bool QUEUE>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_kernel(const PaDecodeArgs a) {
   constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
@@ -227,14 +229,91 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // ---- which (sequence, head, partition): all wave-uniform -----------------------------------------
   const int P = a.max_num_partitions;
   const int Hkv = a.num_kv_heads;
-  const long long wid = blockIdx.x;  // the WAVES waves of a workgroup share one item
-  const int h = (int)(wid % Hkv);
-  const int part = (int)((wid / Hkv) % P);
-  const int b = (int)(wid / ((long long)Hkv * P));
+  // The WAVES waves of a workgroup share one item: (sequence, partition, group of NT 16-row query tiles,
+  // kv head).  The head varies fastest, so the workgroups that stream the same pages (the other heads, and
+  // the other row tiles of the same head, 8 ids apart with 8 kv heads: the same XCD and L2) run together.
+  const int Ge = a.q_len * a.group_size;  // rows per kv head in the buffers
+  const int RT = (Ge + 16 * NT - 1) / (16 * NT);
+
+  // QUEUE: a resident grid of workgroups pulls live items from a counter in the caller's workspace.  Only
+  // partitions a sequence reaches and row tiles that hold real query rows are items, so a ragged batch
+  // launches no workgroup that would exit at once (each of those still costs a wave slot for a
+  // microsecond).  Every workgroup builds, once, the exclusive prefix sum of the per-sequence item counts
+  // in LDS and decodes an item index by binary search in it.
+  __shared__ int q_cum[QUEUE ? kQueueMaxSeqs + 1 : 1];
+  __shared__ int q_ctx[QUEUE ? kQueueMaxSeqs : 1];
+  __shared__ int q_tiles[QUEUE ? kQueueMaxSeqs : 1];
+  __shared__ int q_item;
+  int total_items = 0;
+  if constexpr (QUEUE) {
+    if (wave == 0) {
+      int running = 0;
+      for (int b0 = 0; b0 < a.num_seqs; b0 += 64) {
+        const int bb = b0 + lane;
+        const int c = bb < a.num_seqs ? a.context_lens[bb] : 0;
+        int np = (c + a.partition_size - 1) / a.partition_size;
+        np = np < 0 ? 0 : (np > P ? P : np);
+        const int ql = bb < a.num_seqs ? (a.q_lens ? a.q_lens[bb] : a.q_len) : 0;
+        int tiles = (ql * a.group_size + 16 * NT - 1) / (16 * NT);
+        tiles = tiles > RT ? RT : tiles;
+        const int n = np * tiles;
+        int x = n;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int y = __shfl_up(x, d);
+          if (lane >= d) x += y;
+        }
+        if (bb < a.num_seqs) {
+          q_cum[bb] = running + x - n;
+          q_ctx[bb] = c;
+          q_tiles[bb] = tiles;
+        }
+        running += __builtin_amdgcn_readlane(x, 63);
+      }
+      if (lane == 0) q_cum[a.num_seqs] = running;
+    }
+    __syncthreads();
+    total_items = q_cum[a.num_seqs] * Hkv;
+  }
+
+  for (;;) {  // one pass without the queue
+  int h, rt, b, part, tiles_b = RT;
+  if constexpr (QUEUE) {
+    if (threadIdx.x == 0) q_item = atomicAdd(a.workspace, 1);
+    __syncthreads();
+    const int item = __builtin_amdgcn_readfirstlane(q_item);
+    __syncthreads();  // everybody has read q_item (and is done with the LDS buffers of the previous item)
+    if (item >= total_items) break;
+    h = item % Hkv;
+    const int j = item / Hkv;
+    int lo = 0, hi = a.num_seqs;  // q_cum[lo] <= j < q_cum[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (__builtin_amdgcn_readfirstlane(q_cum[mid]) <= j)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    b = lo;
+    tiles_b = __builtin_amdgcn_readfirstlane(q_tiles[b]);
+    const int local = j - __builtin_amdgcn_readfirstlane(q_cum[b]);
+    part = local / tiles_b;
+    rt = local - part * tiles_b;
+  } else {
+    // The partition index varies slowest: in a ragged batch the partitions that only the longest
+    // sequences reach (workgroups that exit at once for everybody else) come last.
+    const long long wid = blockIdx.x;
+    h = (int)(wid % Hkv);
+    rt = (int)((wid / Hkv) % RT);
+    b = (int)((wid / ((long long)Hkv * RT)) % a.num_seqs);
+    part = (int)(wid / ((long long)Hkv * RT * a.num_seqs));
+  }
+  const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
+  do {  // the body of one item; `break` leaves it
 
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;
-  if (wg_start >= ctx) return;
+  if (wg_start >= ctx) break;
   const int wg_end = min(wg_start + a.partition_size, ctx);
   // this wave's contiguous slice of the partition, in whole steps; a wave past the end idles until the merge
   const int wg_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
@@ -243,9 +322,27 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int part_end = min(part_start + steps_per_wave * kStepTokens, wg_end);
   const bool active = part_start < wg_end;
   const int G = a.group_size;
-  const int Ge = a.q_len * G;  // rows per kv head in the buffers
   const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
   const int rows_valid = qb * G;
+  if (row0 >= rows_valid) {
+    // only padding rows (a ragged batch): nothing to stream; the rows read as "no visible key"
+    if (wave == 0) {
+      const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+      char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                        (int64_t)part * a.stride_tmp_p) * 2;
+      char* op = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+      const bool dir = ctx <= a.partition_size && a.output != nullptr;
+      for (int r = row0 + kg; r < row0 + 16 * NT && r < Ge; r += 4) {
+        if (li == 0) {
+          a.max_logits[eo + r] = -INFINITY;
+          a.exp_sums[eo + r] = 0.f;
+        }
+        *reinterpret_cast<u32x4*>(tp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
+        if (dir) *reinterpret_cast<u32x4*>(op + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
+      }
+    }
+    break;
+  }
 
   // ---- cache addressing -------------------------------------------------------------------------------
   const int log2_bs = 31 - __builtin_clz(a.block_size);
@@ -345,7 +442,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const bool has_alibi = a.alibi_slopes != nullptr;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    int row = 16 * nt + li;
+    int row = row0 + 16 * nt + li;
     int t = row / G;
     limit[nt] = row < rows_valid ? ctx - (qb - 1 - t) : 0;
     slope2[nt] = 0.f;
@@ -361,7 +458,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     const char* q_ptr = (const char*)a.query;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int row = 16 * nt + li;
+      const int row = row0 + 16 * nt + li;
       const bool ok = row < rows_valid;
       const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (ok ? row : 0)) * a.stride_q_h;
 #pragma unroll
@@ -389,7 +486,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   float rscale[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const int row = 16 * nt + li;
+    const int row = row0 + 16 * nt + li;
     float qs = 1.f;
     if (a.query_quant_mode == PA_QUANT_PER_TENSOR) qs = sload_f32(a.query_scale);
     if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row < rows_valid)
@@ -743,19 +840,20 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 
   // ---- epilogue ------------------------------------------------------------------------------------------------
   // max_logits holds the maximum of the scaled logits in the natural-log domain, exp_sums the
-  // un-normalised sum, tmp_output the normalised bf16 partial.  With a single partition per sequence the
+  // un-normalised sum, tmp_output the normalised bf16 partial.  For a sequence that fits in one partition the
   // partial is the result, and it is written to output as well.
   const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
   char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                      (int64_t)part * a.stride_tmp_p) * 2;
-  const bool direct = a.max_num_partitions == 1 && a.output != nullptr;
+  // a sequence that fits in one partition needs no merge: its partial is the result
+  const bool direct = ctx <= a.partition_size && a.output != nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
   const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
   float l_tot[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     l_tot[nt] = quad_row_sum(l_run[nt]);
-    if (16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
+    if (row0 + 16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
       l_tot[nt] = 0.f;
       m_run[nt] = -INFINITY;
     }
@@ -763,15 +861,15 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   if constexpr (WAVES == 1) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int row = 16 * nt + li;
+      const int row = row0 + 16 * nt + li;
       const float inv = l_tot[nt] > 0.f ? v_tensor_scale * acc_unit / l_tot[nt] : 0.f;
       if (row < Ge && kg == 0) {
         a.max_logits[es_off + row] = m_run[nt] * (1.0f / kLog2e);
         a.exp_sums[es_off + row] = l_tot[nt];
       }
-      store_partial_tile(&o_lds[0][0], acc[nt], inv, tmp + (int64_t)(16 * nt) * a.stride_tmp_g * 2,
-                         a.stride_tmp_g * 2, direct ? outp + (int64_t)(16 * nt) * a.stride_out_h * 2 : nullptr,
-                         a.stride_out_h * 2, Ge - 16 * nt, lane);
+      store_partial_tile(&o_lds[0][0], acc[nt], inv, tmp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2,
+                         a.stride_tmp_g * 2, direct ? outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2 : nullptr,
+                         a.stride_out_h * 2, Ge - row0 - 16 * nt, lane);
     }
   } else {
     // merge the waves' (m, l, O): every wave holds the same (row, head dim) in the same lane and register,
@@ -792,17 +890,18 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     constexpr int DBW = 8 / WAVES;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int row = 16 * nt + li;
+      const int lrow = 16 * nt + li;
+      const int row = row0 + lrow;
       float M = -INFINITY;
 #pragma unroll
-      for (int w2 = 0; w2 < WAVES; ++w2) M = fmaxf(M, mg_m[w2][row]);
+      for (int w2 = 0; w2 < WAVES; ++w2) M = fmaxf(M, mg_m[w2][lrow]);
       const float M_safe = M == -INFINITY ? 0.f : M;
       float e[WAVES];
       float L = 0.f;
 #pragma unroll
       for (int w2 = 0; w2 < WAVES; ++w2) {
-        e[w2] = fast_exp2(mg_m[w2][row] - M_safe);
-        L += mg_l[w2][row] * e[w2];
+        e[w2] = fast_exp2(mg_m[w2][lrow] - M_safe);
+        L += mg_l[w2][lrow] * e[w2];
       }
       const float inv = L > 0.f ? v_tensor_scale / L : 0.f;
 #pragma unroll
@@ -825,482 +924,40 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       for (int i = wave; i < 4; i += WAVES) {
         const int r = 4 * i + kg;
         const u32x4 v = *reinterpret_cast<const u32x4*>(&o_lds[0][0] + r * kORowBytes + li * 16);
-        if (r < Ge - 16 * nt) {
-          *reinterpret_cast<u32x4*>(tmp + (int64_t)(16 * nt + r) * a.stride_tmp_g * 2 + li * 16) = v;
-          if (direct) *reinterpret_cast<u32x4*>(outp + (int64_t)(16 * nt + r) * a.stride_out_h * 2 + li * 16) = v;
+        if (r < Ge - row0 - 16 * nt) {
+          *reinterpret_cast<u32x4*>(tmp + (int64_t)(row0 + 16 * nt + r) * a.stride_tmp_g * 2 + li * 16) = v;
+          if (direct)
+            *reinterpret_cast<u32x4*>(outp + (int64_t)(row0 + 16 * nt + r) * a.stride_out_h * 2 + li * 16) = v;
         }
       }
       if (nt + 1 < NT) __syncthreads();
     }
   }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Streaming partition kernel (FP8 cache, FP8 MFMA arithmetic).
-//
-// A fixed grid of resident waves (OCC per SIMD) walks the list of live (sequence, partition, kv head)
-// items round-robin: wave w takes items w, w+W, w+2W, ...  The steps of all of a wave's items form
-// one stream, and the loads of the step after the current one are always in flight, across item
-// boundaries as well, so a wave never drains its memory pipeline between partitions.  The list is
-// never materialised: every workgroup builds the exclusive prefix sum of the per-sequence partition
-// counts (and a copy of the context lengths) in LDS once, and an item index is decoded by a binary
-// search in it.  Stream bookkeeping is wave-uniform (scalar registers, scalar loads).
-// ---------------------------------------------------------------------------------------------
-constexpr int kStreamMaxSeqs = 4096;
-constexpr int kStreamWaves = 4;  // waves per workgroup (they share the two LDS tables, nothing else)
-
-struct StepDesc {
-  int valid;
-  int b, h, part;
-  int ctx;       // context length of the sequence
-  int tok0;      // first token of the step
-  int part_end;  // one past the last live token of the partition
-  int first;     // first step of its item
-  int last;      // last step of its item
-  long long item;
-};
-
-struct StepPages {
-  int p[4];    // page of each 16-token tile of the step
-  int off[4];  // token offset of the tile inside its page
-};
-
-template <int NT, bool PER_TOKEN, bool BS16, int OCC>
-__global__ __launch_bounds__(64 * kStreamWaves) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
-void pa_partition_stream_kernel(const PaDecodeArgs a) {
-  constexpr int KVT = PA_DTYPE_FP8_E4M3FN;
-  typedef StepData<KVT, PER_TOKEN> SD;
-
-  __shared__ int cum_lds[kStreamMaxSeqs + 1];  // partitions of all earlier sequences
-  __shared__ int ctx_lds[kStreamMaxSeqs];
-  __shared__ __attribute__((aligned(16))) char o_lds[kStreamWaves][16 * kORowBytes];
-
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int li = lane & 15;
-  const int kg = lane >> 4;
-  const int B = a.num_seqs;
-  const int Hkv = a.num_kv_heads;
-  const int ps = a.partition_size;
-  const int G = a.group_size;
-  const int Ge = a.q_len * G;
-
-  // ---- item table: wave 0 scans the context lengths ------------------------------------------------------
-  if (wave == 0) {
-    int running = 0;
-    for (int b0 = 0; b0 < B; b0 += 64) {
-      const int bb = b0 + lane;
-      const int c = bb < B ? a.context_lens[bb] : 0;
-      int n = (c + ps - 1) / ps;
-      n = n < 0 ? 0 : (n > a.max_num_partitions ? a.max_num_partitions : n);
-      int x = n;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const int y = __shfl_up(x, d);
-        if (lane >= d) x += y;
+  if constexpr (QUEUE) {
+    // rows of padding query positions beyond the last real tile: this workgroup fills them
+    if (rt == tiles_b - 1 && wave == 0) {
+      for (int r = 16 * NT * tiles_b + kg; r < Ge; r += 4) {
+        if (li == 0) {
+          a.max_logits[es_off + r] = -INFINITY;
+          a.exp_sums[es_off + r] = 0.f;
+        }
+        *reinterpret_cast<u32x4*>(tmp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
+        if (direct) *reinterpret_cast<u32x4*>(outp + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
       }
-      if (bb < B) {
-        cum_lds[bb] = running + x - n;
-        ctx_lds[bb] = c;
-      }
-      running += __builtin_amdgcn_readlane(x, 63);
     }
-    if (lane == 0) cum_lds[B] = running;
   }
-  __syncthreads();
-  const long long total_items = (long long)cum_lds[B] * Hkv;
-  const long long W = (long long)gridDim.x * kStreamWaves;
-  const long long w = (long long)blockIdx.x * kStreamWaves + wave;
-  if (w >= total_items) return;
-
-  auto lds_i32 = [&](const int* tab, int idx) { return __builtin_amdgcn_readfirstlane(tab[idx]); };
-
-  // ---- stream cursor -----------------------------------------------------------------------------------------
-  auto decode_item = [&](long long i) {
-    StepDesc d;
-    d.valid = 1;
-    d.item = i;
-    d.h = (int)(i % Hkv);
-    const int j = (int)(i / Hkv);
-    int lo = 0, hi = B;  // cum[lo] <= j < cum[hi]
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (lds_i32(cum_lds, mid) <= j)
-        lo = mid;
-      else
-        hi = mid;
-    }
-    d.b = lo;
-    d.part = j - lds_i32(cum_lds, lo);
-    d.ctx = lds_i32(ctx_lds, lo);
-    d.tok0 = d.part * ps;
-    const int pe = d.tok0 + ps;
-    d.part_end = pe < d.ctx ? pe : d.ctx;
-    d.first = 1;
-    d.last = d.tok0 + kStepTokens >= d.part_end;
-    return d;
-  };
-  auto advance = [&](const StepDesc& d) {
-    StepDesc n = d;
-    if (!d.valid) return n;
-    if (!d.last) {
-      n.tok0 = d.tok0 + kStepTokens;
-      n.first = 0;
-      n.last = n.tok0 + kStepTokens >= n.part_end;
-      return n;
-    }
-    const long long i = d.item + W;
-    if (i >= total_items) {
-      n.valid = 0;
-      n.first = 0;
-      n.last = 0;
-      return n;
-    }
-    return decode_item(i);
-  };
-
-  // ---- cache addressing ------------------------------------------------------------------------------------------
-  const int log2_bs = 31 - __builtin_clz(a.block_size);
-  const int bs_mask = a.block_size - 1;
-  const int64_t k_block_bytes = a.stride_k_b;
-  const int64_t v_block_bytes = a.stride_v_b;
-  const uint32_t k_chunk_bytes = BS16 ? 256u : (uint32_t)a.stride_k_c;
-  uint32_t k_lane_off[2];
-#pragma unroll
-  for (int ld = 0; ld < 2; ++ld) k_lane_off[ld] = (uint32_t)(kg * k_chunk_bytes + li * 16) + 4 * ld * k_chunk_bytes;
-  const bool vt = a.v_transposed;
-  const uint32_t v_row_bytes = BS16 ? 16u : (vt ? 16u : (uint32_t)a.stride_v_2);
-  const int64_t v_tile_bytes = BS16 ? 16 : (vt ? a.stride_v_2 : 16);
-  uint32_t v_lane_off[8];
-#pragma unroll
-  for (int db = 0; db < 8; ++db) v_lane_off[db] = li * v_row_bytes + 16 * db * v_row_bytes;
-
-  auto load_pages = [&](const StepDesc& d) {
-    StepPages pg;
-    if (d.valid) {
-      const int* bt = a.block_tables + (int64_t)d.b * a.stride_bt_s;
-      const int last_tile_tok = (d.part_end - 1) & ~15;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int t = d.tok0 + 16 * j;
-        t = t > last_tile_tok ? last_tile_tok : t;
-        pg.p[j] = sload_i32(bt + (t >> log2_bs));
-        pg.off[j] = t & bs_mask;
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) pg.p[j] = pg.off[j] = 0;  // page 0: requested, never used
-    }
-    return pg;
-  };
-  auto issue_k = [&](SD& sd, int h, const StepPages& pg) {
-    const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const char* tb = kbase + (int64_t)pg.p[j] * k_block_bytes + (int64_t)pg.off[j] * 16;
-#pragma unroll
-      for (int ld = 0; ld < 2; ++ld) sd.k[j][ld] = load16(tb + k_lane_off[ld]);
-      if constexpr (PER_TOKEN) {
-        const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + (int64_t)h * a.stride_kvscale_h + pg.off[j] + 4 * kg;
-        sd.ks[j] = *reinterpret_cast<const f32x4*>(a.key_scale + so);
+  } while (0);
+  if constexpr (!QUEUE) break;
+  }  // for (;;)
+  if constexpr (QUEUE) {
+    // the last workgroup out leaves the workspace as it found it: zero
+    if (threadIdx.x == 0) {
+      __threadfence();
+      if (atomicAdd(a.workspace + 1, 1) == (int)gridDim.x - 1) {
+        a.workspace[0] = 0;
+        a.workspace[1] = 0;
       }
     }
-  };
-  auto issue_v = [&](SD& sd, int h, const StepPages& pg) {
-    const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h;
-    const int page = kg == 0 ? pg.p[0] : (kg == 1 ? pg.p[1] : (kg == 2 ? pg.p[2] : pg.p[3]));
-    const int off = kg == 0 ? pg.off[0] : (kg == 1 ? pg.off[1] : (kg == 2 ? pg.off[2] : pg.off[3]));
-    const char* tb = vbase + (int64_t)page * v_block_bytes + (int64_t)(off >> 4) * v_tile_bytes;
-#pragma unroll
-    for (int db = 0; db < 8; ++db) sd.v[db][0] = load16(tb + v_lane_off[db]);
-    if constexpr (PER_TOKEN) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + (int64_t)h * a.stride_kvscale_h + pg.off[j] + 4 * kg;
-        sd.vs[j] = *reinterpret_cast<const f32x4*>(a.value_scale + so);
-      }
-    }
-  };
-
-  // ---- the stream starts: first step's data, then the descriptors of the next two steps ------------------------
-  SD sd;
-  StepDesc d0 = decode_item(w);
-  {
-    const StepPages pg0 = load_pages(d0);
-    issue_k(sd, d0.h, pg0);
-    issue_v(sd, d0.h, pg0);
-  }
-  StepDesc d1 = advance(d0);
-  StepPages pg1 = load_pages(d1);
-
-  float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
-  if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
-    k_tensor_scale = sload_f32(a.key_scale);
-    v_tensor_scale = sload_f32(a.value_scale);
-  }
-  const float scale2 = a.softmax_scale * k_tensor_scale * kLog2e;
-  const bool has_alibi = a.alibi_slopes != nullptr;
-
-  // per-item, per-lane state
-  int limit[NT];
-  float slope2[NT], rscale[NT];
-  i32x8 qhi[NT], qlo[NT];
-  float m_run[NT], l_run[NT];
-  f32x4 acc[NT][8];
-  float v_run = 1e-30f;
-  int rows_valid = 0, min_limit = 0;
-
-  auto begin_item = [&](const StepDesc& d) {
-    const int qb = a.q_lens ? sload_i32(a.q_lens + d.b) : a.q_len;
-    rows_valid = qb * G;
-    min_limit = d.ctx - (qb - 1);
-    const char* q_ptr = (const char*)a.query;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int row = 16 * nt + li;
-      const bool ok = row < rows_valid;
-      const int t = row / G;
-      limit[nt] = ok ? d.ctx - (qb - 1 - t) : 0;
-      slope2[nt] = 0.f;
-      if (has_alibi && ok) slope2[nt] = a.alibi_slopes[d.h * G + (row - t * G)] * kLog2e;
-      float qs = 1.f;
-      if (a.query_quant_mode == PA_QUANT_PER_TENSOR) qs = sload_f32(a.query_scale);
-      if (a.query_quant_mode == PA_QUANT_PER_TOKEN && ok)
-        qs = a.query_scale[(int64_t)d.b * a.stride_qscale_s + d.h * Ge + row];
-      const int64_t e0 = (int64_t)d.b * a.stride_q_s + (int64_t)(d.h * Ge + (ok ? row : 0)) * a.stride_q_h;
-      if (a.query_dtype == PA_DTYPE_BF16) {
-        // q * cq = hi + lo with hi, lo in e4m3 (|q * cq| <= 224); the logits are divided by cq again
-        float f[32];
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const u32x4 raw = load16(q_ptr + (e0 + 64 * c + 16 * kg + 8 * half) * 2);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              f[16 * c + 8 * half + 2 * e] = bf16_bits_to_f32(raw[e] & 0xffffu);
-              f[16 * c + 8 * half + 2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
-            }
-          }
-        }
-        float amax = 0.f;
-#pragma unroll
-        for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(f[e]));
-        amax = quad_row_max(amax);
-        const float cq = amax > 0.f ? 224.f / amax : 1.f;
-        qs *= amax > 0.f ? amax * (1.f / 224.f) : 1.f;
-#pragma unroll
-        for (int wd = 0; wd < 8; ++wd) {
-          const float x0 = f[4 * wd] * cq, x1 = f[4 * wd + 1] * cq, x2 = f[4 * wd + 2] * cq, x3 = f[4 * wd + 3] * cq;
-          int hi = 0, lo = 0;
-          hi = __builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, hi, false);
-          hi = __builtin_amdgcn_cvt_pk_fp8_f32(x2, x3, hi, true);
-          const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
-          const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
-          lo = __builtin_amdgcn_cvt_pk_fp8_f32(x0 - b01[0], x1 - b01[1], lo, false);
-          lo = __builtin_amdgcn_cvt_pk_fp8_f32(x2 - b23[0], x3 - b23[1], lo, true);
-          qhi[nt][wd] = ok ? hi : 0;
-          qlo[nt][wd] = ok ? lo : 0;
-        }
-      } else {
-        // FP8 query: the bytes are the operand
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const u32x4 raw = load16(q_ptr + e0 + 64 * c + 16 * kg);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            qhi[nt][4 * c + e] = ok ? (int)raw[e] : 0;
-            qlo[nt][4 * c + e] = 0;
-          }
-        }
-      }
-      rscale[nt] = scale2 * qs;
-      m_run[nt] = -INFINITY;
-      l_run[nt] = 0.f;
-#pragma unroll
-      for (int db = 0; db < 8; ++db) acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    v_run = 1e-30f;
-  };
-
-  auto end_item = [&](const StepDesc& d) {
-    const int64_t es_off = (int64_t)d.b * a.stride_es_s + (int64_t)d.h * a.stride_es_h + (int64_t)d.part * a.stride_es_p;
-    char* tmp = (char*)a.tmp_output + ((int64_t)d.b * a.stride_tmp_s + (int64_t)d.h * a.stride_tmp_h +
-                                       (int64_t)d.part * a.stride_tmp_p) * 2;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      float l = quad_row_sum(l_run[nt]);
-      const int row = 16 * nt + li;
-      float m_out = m_run[nt] * (1.0f / kLog2e);
-      if (row >= rows_valid) {  // padding rows of a ragged batch: no visible key
-        l = 0.f;
-        m_out = -INFINITY;
-      }
-      float inv = l > 0.f ? v_tensor_scale / l : 0.f;
-      inv *= (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f);
-      if (row < Ge) {
-        if (kg == 0) {
-          a.max_logits[es_off + row] = m_out;
-          a.exp_sums[es_off + row] = l;
-        }
-      }
-      store_partial_tile(&o_lds[wave][0], acc[nt], inv, tmp + (int64_t)(16 * nt) * a.stride_tmp_g * 2,
-                         a.stride_tmp_g * 2, nullptr, 0, Ge - 16 * nt, lane);
-    }
-  };
-
-  // ---- one step; the next step's K and V are requested as this step's are consumed ---------------------------
-  auto step = [&]<bool FULL>(int tok0, int ctx, int h_next, const StepPages& pg_next) {
-    f32x4 s[NT][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const i32x8 ka = {(int)sd.k[j][0][0], (int)sd.k[j][0][1], (int)sd.k[j][0][2], (int)sd.k[j][0][3],
-                        (int)sd.k[j][1][0], (int)sd.k[j][1][1], (int)sd.k[j][1][2], (int)sd.k[j][1][3]};
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        s[nt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi[nt], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-        s[nt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo[nt], s[nt][j], 0, 0, 0, 0, 0, 0);
-      }
-    }
-    f32x4 ks_cur[PER_TOKEN ? 4 : 1], vs_cur[PER_TOKEN ? 4 : 1];
-    if constexpr (PER_TOKEN) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ks_cur[j] = sd.ks[j];
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    issue_k(sd, h_next, pg_next);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // per-token V scales: P carries v_scale / v_run (<= 1); the accumulator is in units of v_run
-    float vfac = 1.f, pmul = 256.f;
-    if constexpr (PER_TOKEN) {
-      float vmx = 0.f;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        vs_cur[j] = sd.vs[j];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          if constexpr (!FULL) {
-            const int col = tok0 + 16 * j + 4 * kg + r;
-            vs_cur[j][r] = col < ctx ? vs_cur[j][r] : 0.f;
-          }
-          vmx = fmaxf(vmx, vs_cur[j][r]);
-        }
-      }
-      vmx = quad_row_max(vmx);
-      const float v_new = fmaxf(v_run, vmx);
-      vfac = v_run / v_new;
-      pmul = 256.f / v_new;
-      v_run = v_new;
-    }
-    uint32_t ph[NT][4], pl[NT][4];  // P head / residual, 4 tokens per dword
-
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const float rs = rscale[nt];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v = s[nt][j][r] * rs;
-          if constexpr (PER_TOKEN) v *= ks_cur[j][r];
-          if constexpr (!FULL) {
-            const int col = tok0 + 16 * j + 4 * kg + r;
-            v += slope2[nt] * (float)(col - ctx + 1);
-            v = col < limit[nt] ? v : -INFINITY;
-          }
-          s[nt][j][r] = v;
-          mx = fmaxf(mx, v);
-        }
-      }
-      mx = quad_row_max(mx);
-      const float m_new = fmaxf(m_run[nt], mx);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
-      m_run[nt] = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float p0 = fast_exp2(s[nt][j][0] - m_safe);
-        float p1 = fast_exp2(s[nt][j][1] - m_safe);
-        float p2 = fast_exp2(s[nt][j][2] - m_safe);
-        float p3 = fast_exp2(s[nt][j][3] - m_safe);
-        psum += (p0 + p1) + (p2 + p3);
-        if constexpr (PER_TOKEN) {
-          p0 *= vs_cur[j][0];
-          p1 *= vs_cur[j][1];
-          p2 *= vs_cur[j][2];
-          p3 *= vs_cur[j][3];
-        }
-        p0 *= pmul;
-        p1 *= pmul;
-        p2 *= pmul;
-        p3 *= pmul;
-        int hi = 0, lo = 0;
-        hi = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, hi, false);
-        hi = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, hi, true);
-        const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
-        const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
-        lo = __builtin_amdgcn_cvt_pk_fp8_f32(p0 - b01[0], p1 - b01[1], lo, false);
-        lo = __builtin_amdgcn_cvt_pk_fp8_f32(p2 - b23[0], p3 - b23[1], lo, true);
-        ph[nt][j] = (uint32_t)hi;
-        pl[nt][j] = (uint32_t)lo;
-      }
-      l_run[nt] = l_run[nt] * alpha + psum;
-      const float alpha_acc = alpha * vfac;
-#pragma unroll
-      for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha_acc;
-    }
-
-    if constexpr (!FULL) {
-      // zero the V bytes of tokens at or beyond ctx (stale cache contents may decode to NaN)
-      int nvalid = ctx - (tok0 + 16 * kg);
-      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
-#pragma unroll
-      for (int db = 0; db < 8; ++db) sd.v[db][0] = keep_first_bytes(sd.v[db][0], nvalid);
-    }
-
-    // B operand of O^T += V^T P^T: lane group kg must hold all 16 tokens of tile kg
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      quad_transpose(ph[nt]);
-      quad_transpose(pl[nt]);
-    }
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-#pragma unroll
-      for (int db = 0; db < 8; ++db) {
-        const long va = (long)(((uint64_t)sd.v[db][0][2 * hf + 1] << 32) | sd.v[db][0][2 * hf]);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const long bh = (long)(((uint64_t)ph[nt][2 * hf + 1] << 32) | ph[nt][2 * hf]);
-          const long bl = (long)(((uint64_t)pl[nt][2 * hf + 1] << 32) | pl[nt][2 * hf]);
-          acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(va, bh, acc[nt][db], 0, 0, 0);
-          acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(va, bl, acc[nt][db], 0, 0, 0);
-        }
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    issue_v(sd, h_next, pg_next);
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  // ---- the stream ------------------------------------------------------------------------------------------------
-  while (true) {
-    const StepDesc d2 = advance(d1);
-    const StepPages pg2 = load_pages(d2);
-    if (d0.first) begin_item(d0);
-    const bool full = !has_alibi && d0.tok0 + kStepTokens <= min_limit;
-    if (full)
-      step.template operator()<true>(d0.tok0, d0.ctx, d1.h, pg1);
-    else
-      step.template operator()<false>(d0.tok0, d0.ctx, d1.h, pg1);
-    if (d0.last) end_item(d0);
-    if (!d1.valid) break;
-    d0 = d1;
-    d1 = d2;
-    pg1 = pg2;
   }
 }
 
@@ -1309,6 +966,7 @@ void pa_partition_stream_kernel(const PaDecodeArgs a) {
 // (m_p, l_p); the weights w_p = l_p e^{m_p - M} are broadcast with v_readlane while the partial
 // outputs of the chunk stream in, eight loads in flight per lane.
 // ---------------------------------------------------------------------------------------------
+template <bool SKIP_SINGLE>
 __global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
   const int lane = threadIdx.x & 63;
   const int Ge = a.q_len * a.group_size;
@@ -1326,6 +984,8 @@ __global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
 
   uint32_t* out = reinterpret_cast<uint32_t*>((char*)a.output +
                                               ((int64_t)b * a.stride_out_s + (int64_t)(h * Ge + row) * a.stride_out_h) * 2) + lane;
+  // SKIP_SINGLE: the partition kernel of the same call has written the rows of sequences with one partition
+  if (SKIP_SINGLE && n == 1) return;
   if (n <= 0 || row >= qb * a.group_size) {
     *out = 0u;
     return;
@@ -1407,22 +1067,7 @@ int check_common(const PaDecodeArgs* a) {
     return PA_ERR_BAD_SHAPE;
   if (a->partition_size <= 0 || a->partition_size % 256) return PA_ERR_BAD_SHAPE;
   if (a->head_size != kHeadSize) return PA_ERR_UNSUPPORTED;
-  if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;
-  return PA_OK;
-}
-
-template <int NT, int KVT, bool PT, bool FP8MATH, bool BS16, int W>
-int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
-  constexpr int OCC = NT == 1 ? 2 : 1;
-  constexpr int DEPTH = 1;
-  const long long blocks = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
-  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, FP8MATH, BS16, W, OCC, DEPTH>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
+  if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;  // the reference's limit
   return PA_OK;
 }
 
@@ -1436,15 +1081,33 @@ int device_num_cus() {
   return n;
 }
 
-template <int NT, bool PT, bool BS16>
-int launch_stream(const PaDecodeArgs& a, hipStream_t stream) {
+// The queued launch is used when the caller gave a workspace and per-sequence query lengths (row tiles of
+// padding rows are then common): a resident grid pulls live items from a counter.  Without query lengths
+// the only workgroups with nothing to do are partitions past a sequence's end, which the plain launch
+// orders last; there the queue's bookkeeping costs more than it saves (measured: +10 % on a uniform batch).
+bool use_queue(const PaDecodeArgs& a) {
+  static const bool off = [] {
+    const char* e = getenv("PA_DECODE_QUEUE");
+    return e && e[0] == '0';
+  }();
+  return !off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr;
+}
+
+template <int NT, int KVT, bool PT, bool FP8MATH, bool BS16, int W>
+int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   constexpr int OCC = NT == 1 ? 2 : 1;
-  const long long max_items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
-  long long blocks = (long long)device_num_cus() * 4 * OCC / kStreamWaves;
-  const long long need = (max_items + kStreamWaves - 1) / kStreamWaves;
-  blocks = blocks < need ? blocks : need;
-  hipLaunchKernelGGL((pa_partition_stream_kernel<NT, PT, BS16, OCC>), dim3((unsigned)blocks), dim3(64 * kStreamWaves), 0,
-                     stream, a);
+  constexpr int DEPTH = 1;
+  const int ge = a.q_len * a.group_size;
+  const int row_tiles = (ge + 16 * NT - 1) / (16 * NT);
+  const long long blocks = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * row_tiles;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  if (use_queue(a)) {
+    long long resident = (long long)device_num_cus() * 4 * OCC / W;
+    resident = resident < blocks ? resident : blocks;
+    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, FP8MATH, BS16, W, OCC, DEPTH, true>), dim3((unsigned)resident),
+                       dim3(64 * W), 0, stream, a);
+  } else
+  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, FP8MATH, BS16, W, OCC, DEPTH, false>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
@@ -1453,24 +1116,18 @@ int launch_stream(const PaDecodeArgs& a, hipStream_t stream) {
   return PA_OK;
 }
 
-template <bool PT, bool BS16>
-int launch_stream_nt(const PaDecodeArgs& a, int nt, hipStream_t stream) {
-  switch (nt) {
-    case 1: return launch_stream<1, PT, BS16>(a, stream);
-    case 2: return launch_stream<2, PT, BS16>(a, stream);
-    case 3:
-    case 4: return launch_stream<4, PT, BS16>(a, stream);
-  }
-  return PA_ERR_UNSUPPORTED;
-}
 
-// The streaming kernel is opt-in (PA_DECODE_STREAM=1): for FP8 caches and at most kStreamMaxSeqs sequences.
-bool use_stream_kernel(const PaDecodeArgs& a) {
-  static const bool on = [] {
-    const char* e = getenv("PA_DECODE_STREAM");
-    return e && e[0] == '1';
+// 16-row query tiles per workgroup.  More than 16 query rows per kv head (large GQA groups, MTP) are split
+// over workgroups of one tile each by default: they re-read the same pages at the same time from the
+// same L2, run the 2-waves-per-SIMD variant, and tiles that hold only padding rows cost nothing.
+// PA_DECODE_TILES=2 keeps two tiles in one workgroup (one pass over the pages, 1 wave per SIMD).
+int tiles_per_workgroup(int total_tiles) {
+  static const int forced = [] {
+    const char* e = getenv("PA_DECODE_TILES");
+    return e ? atoi(e) : 0;
   }();
-  return on && a.kv_dtype == PA_DTYPE_FP8_E4M3FN && a.num_seqs <= kStreamMaxSeqs;
+  const int t = forced == 2 ? 2 : 1;
+  return t < total_tiles ? t : total_tiles;
 }
 
 // Waves per workgroup: about 256 tokens (4 steps) per wave at least, and at most 4 / NT waves (the
@@ -1498,10 +1155,31 @@ int launch_partition_nt(const PaDecodeArgs& a, int nt, hipStream_t stream) {
     case 2:
       if (w == 2) return launch_partition_w<2, KVT, PT, FP8MATH, BS16, 2>(a, stream);
       return launch_partition_w<2, KVT, PT, FP8MATH, BS16, 1>(a, stream);
-    case 3:
-    case 4: return launch_partition_w<4, KVT, PT, FP8MATH, BS16, 1>(a, stream);
   }
   return PA_ERR_UNSUPPORTED;
+}
+
+int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!a->output) return PA_ERR_NULL_POINTER;
+  if (a->stride_out_h % 2 || a->stride_out_s % 2 || a->stride_tmp_g % 2 || a->stride_tmp_p % 2 ||
+      a->stride_tmp_h % 2 || a->stride_tmp_s % 2)
+    return PA_ERR_BAD_SHAPE;
+  const long long rows = (long long)a->num_seqs * a->num_kv_heads * a->q_len * a->group_size;
+  const long long blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  if (skip_single)
+    hipLaunchKernelGGL(pa_reduce_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
+  else
+    hipLaunchKernelGGL(pa_reduce_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return PA_OK;
 }
 
 }  // namespace
@@ -1532,12 +1210,14 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   if (num_cus <= 0) num_cus = device_num_cus();
   // The fewest partitions per sequence that still give every wave slot of the GPU a wave: each extra
   // partition costs a (rows x 128) bf16 partial written and read back plus the merge, and a single
-  // partition needs no second kernel at all.  A workgroup splits its partition over up to 4 / NT waves
-  // (at least 256 tokens each); no wave is given more than 2048 tokens, which keeps ragged batches balanced.
-  const int nt = (rows_per_group + 15) / 16;
-  const int cap_w = nt <= 1 ? 4 : (nt == 2 ? 2 : 1);
+  // partition needs no second kernel at all.  A workgroup (one 16-row query tile) splits its partition over
+  // up to 4 waves (at least 256 tokens each); no wave is given more than 2048 tokens, which keeps ragged
+  // batches balanced.
+  const int total_tiles = (rows_per_group + 15) / 16;
+  const int nt = tiles_per_workgroup(total_tiles);
+  const int cap_w = nt <= 1 ? 4 : 2;
   const long long slots = (long long)num_cus * 4 * (nt <= 1 ? 2 : 1);
-  const long long rows = (long long)num_seqs * num_kv_heads;
+  const long long rows = (long long)num_seqs * num_kv_heads * ((total_tiles + nt - 1) / nt);
   for (int parts = 1;; ++parts) {
     int ps = (max_context_len + parts - 1) / parts;
     ps = (ps + 255) / 256 * 256;
@@ -1577,17 +1257,13 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
     return PA_ERR_BAD_SHAPE;
 
   const int Ge = a->q_len * a->group_size;
-  const int nt = (Ge + 15) / 16;
+  const int nt = tiles_per_workgroup((Ge + 15) / 16);
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   const bool pt = a->kv_quant_mode == PA_QUANT_PER_TOKEN;
   if (a->kv_dtype == PA_DTYPE_FP8_E4M3FN) {
     // constant in-page strides: block size 16 with the default dense layout
     const bool bs16 = a->block_size == 16 && a->stride_k_c == 256 &&
                       (a->v_transposed ? a->stride_v_2 == 2048 : a->stride_v_2 == 16);
-    if (use_stream_kernel(*a)) {
-      if (bs16) return pt ? launch_stream_nt<true, true>(*a, nt, stream) : launch_stream_nt<false, true>(*a, nt, stream);
-      return pt ? launch_stream_nt<true, false>(*a, nt, stream) : launch_stream_nt<false, false>(*a, nt, stream);
-    }
     if (bs16)
       return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true, true>(*a, nt, stream)
                 : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true, true>(*a, nt, stream);
@@ -1598,33 +1274,15 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
   return launch_partition_nt<PA_DTYPE_BF16, false, false, false>(*a, nt, stream);
 }
 
-int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
-  int rc = check_common(a);
-  if (rc) return rc;
-  if (!a->output) return PA_ERR_NULL_POINTER;
-  if (a->stride_out_h % 2 || a->stride_out_s % 2 || a->stride_tmp_g % 2 || a->stride_tmp_p % 2 ||
-      a->stride_tmp_h % 2 || a->stride_tmp_s % 2)
-    return PA_ERR_BAD_SHAPE;
-  const long long rows = (long long)a->num_seqs * a->num_kv_heads * a->q_len * a->group_size;
-  const long long blocks = (rows + 3) / 4;
-  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-  hipLaunchKernelGGL(pa_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
-}
+int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) { return launch_reduce(a, hip_stream, false); }
 
 int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
   if (a && a->struct_size == sizeof(PaDecodeArgs) && !a->output) return PA_ERR_NULL_POINTER;
   int rc = pa_decode_partition(a, hip_stream);
   if (rc) return rc;
-  // with one partition per sequence the partition kernel has written output itself
-  if (a->max_num_partitions == 1 && !use_stream_kernel(*a)) return PA_OK;
-  return pa_decode_reduce(a, hip_stream);
+  // the partition kernel has written the rows of every sequence that fits in one partition itself
+  if (a->max_num_partitions == 1) return PA_OK;
+  return launch_reduce(a, hip_stream, true);
 }
 
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream) {

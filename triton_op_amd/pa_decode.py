@@ -12,7 +12,9 @@ pa_decode_triton.py:523-685.  Differences, all additive:
   nothing is allocated;
 * `partition_size` may be any multiple of 256 (the reference's constant); by default the tuning
   layer picks it from the batch shape and the longest context;
-* `query_lens` gives a per-sequence number of new tokens (ragged MTP batches).
+* `query_lens` gives a per-sequence number of new tokens (ragged MTP batches);
+* `workspace` is a zeroed int32 tensor of 64 bytes holding a work-item counter for ragged batches (one is
+  allocated per call/plan when it is not given; calls that may overlap on the GPU need one each).
 
 There is no eager/torch implementation behind this function: without the HIP library it raises.
 """
@@ -102,6 +104,7 @@ def plan_decode(
     tmp_output: Optional[torch.Tensor] = None,
     partition_size: Optional[int] = None,
     query_lens: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None,
 ) -> DecodePlan:
     # ---- shapes (pa_decode_triton_gluon_fp8.py:1703-1722) ------------------------------------
     if output.dim() != 3:
@@ -275,6 +278,13 @@ def plan_decode(
     a.value_scale = _ptr(value_scale) if kv_mode != _cabi.PA_QUANT_NONE else None
     a.alibi_slopes = _ptr(alibi_slopes)
     a.exp_sums, a.max_logits, a.tmp_output = exp_sums.data_ptr(), max_logits.data_ptr(), tmp_output.data_ptr()
+    # zeroed work-item counter for ragged batches; the kernels leave it zero, so the plan can be replayed
+    if workspace is None:
+        workspace = torch.zeros(_cabi.PA_DECODE_WORKSPACE_BYTES // 4, dtype=torch.int32, device=dev)
+    elif workspace.dtype != torch.int32 or workspace.numel() * 4 < _cabi.PA_DECODE_WORKSPACE_BYTES or \
+            not workspace.is_contiguous() or workspace.device != dev:
+        raise ValueError(f"workspace must be a contiguous int32 tensor of >= {_cabi.PA_DECODE_WORKSPACE_BYTES} bytes on {dev}")
+    a.workspace = workspace.data_ptr()
     a.num_seqs, a.num_kv_heads, a.group_size, a.q_len = num_seqs, num_kv_heads, group, q_len
     a.head_size, a.block_size = head_size, block_size
     a.max_num_partitions, a.partition_size = max_parts, partition_size
@@ -291,7 +301,7 @@ def plan_decode(
     a.stride_tmp_s, a.stride_tmp_h, a.stride_tmp_p, a.stride_tmp_g = (tmp_output.stride(i) for i in range(4))
     a.stride_qscale_s, a.stride_kvscale_b, a.stride_kvscale_h = stride_qs, stride_kvs_b, stride_kvs_h
     keep = (output, query, key_cache, value_cache, sequence_lengths, block_tables, query_scale, key_scale,
-            value_scale, alibi_slopes, query_lens)
+            value_scale, alibi_slopes, query_lens, workspace)
     return DecodePlan(a, keep, exp_sums, max_logits, tmp_output, output)
 
 
@@ -317,6 +327,7 @@ def paged_attention_decode(
     tmp_output: Optional[torch.Tensor] = None,
     partition_size: Optional[int] = None,
     query_lens: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None,
 ) -> Dict[str, object]:
     """Split-KV paged-attention decode; writes `output` in place on torch's current stream and
     returns the partition buffers under the reference's keys."""
@@ -324,7 +335,7 @@ def paged_attention_decode(
         output, query, key_cache, value_cache, sequence_lengths, block_tables, softmax_scale,
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
         num_sequence_partitions, alibi_slopes, exp_sums=exp_sums, max_logits=max_logits,
-        tmp_output=tmp_output, partition_size=partition_size, query_lens=query_lens)
+        tmp_output=tmp_output, partition_size=partition_size, query_lens=query_lens, workspace=workspace)
     plan.run()
     return {
         "temporary_output": plan.tmp_output,
