@@ -80,6 +80,7 @@ typedef struct PaDecodeArgs {
   const float* key_scale;     /* optional */
   const float* value_scale;   /* optional */
   const float* alibi_slopes;  /* optional, [Hkv*G] */
+  const float* sinks;         /* optional, [Hkv*Ge]: attention-sink logit of every query row (natural-log domain) */
   float* exp_sums;
   float* max_logits;
   void* tmp_output;

@@ -158,6 +158,7 @@ def masked_attention(
     output_dtype: torch.dtype,
     is_causal: bool = True,
     alibi_slopes: Optional[torch.Tensor] = None,  # [Hq]
+    sinks: Optional[torch.Tensor] = None,  # [q, Hq] attention-sink logits
 ) -> torch.Tensor:
     hq, hkv = query.shape[1], key.shape[1]
     key = key.repeat_interleave(hq // hkv, dim=1)
@@ -173,7 +174,13 @@ def masked_attention(
         keep = torch.ones(qlen, klen, dtype=torch.bool).tril(diagonal=klen - qlen)
         bias.masked_fill_(keep.logical_not(), float("-inf"))
         scores = scores + bias
-    weights = torch.softmax(scores, dim=-1)
+    if sinks is not None:
+        # pa_decode_triton_gluon_fp8.py:1118-1123: exp(sink - max) joins the denominator, no value attached:
+        # a key column with that logit whose value row is zero
+        scores = torch.cat([scores, sinks.float().t().unsqueeze(-1)], dim=-1)
+        weights = torch.softmax(scores, dim=-1)[..., :-1]
+    else:
+        weights = torch.softmax(scores, dim=-1)
     out = torch.einsum("hqk,khd->qhd", weights.float(), value.float())
     return out.to(output_dtype)
 
@@ -239,6 +246,7 @@ def paged_attention_decode_oracle(
     seq_ids: Optional[Sequence[int]] = None,
     query_scale: Optional[torch.Tensor] = None,
     q_max: Optional[int] = None,
+    sinks: Optional[torch.Tensor] = None,  # [Hkv*qmax*G], one logit per packed query row
 ) -> torch.Tensor:
     """The oracle behind the entry point's own conventions: output [B, Hkv*qmax*G, D] in
     query's 16-bit dtype (bf16 when the query is FP8).  Rows of padded query positions
@@ -263,7 +271,10 @@ def paged_attention_decode_oracle(
         k, v = gather_sequence(key_flat, value_flat, ks, vs, block_tables[b], ctx, bs)
         # [Hkv, qmax, G, D] -> token-major [qb, Hq, D]
         qv = qf[b].view(hkv, qmax, g, d)[:, :qb].permute(1, 0, 2, 3).reshape(qb, hkv * g, d)
-        o = masked_attention(qv, k, v, softmax_scale, torch.float32, True, alibi_slopes)
+        sk = None
+        if sinks is not None:
+            sk = sinks.float().view(hkv, qmax, g)[:, :qb].permute(1, 0, 2).reshape(qb, hkv * g)
+        o = masked_attention(qv, k, v, softmax_scale, torch.float32, True, alibi_slopes, sk)
         o = o.view(qb, hkv, g, d).permute(1, 0, 2, 3)  # [Hkv, qb, G, D]
         out[b].view(hkv, qmax, g, d)[:, :qb] = o.to(out_dtype)
     return out

@@ -229,3 +229,15 @@ def test_golden_fixtures_match_oracle():
             case["query"], case["key_cache"], case["value_cache"], case["context_lens"], case["block_tables"],
             case["softmax_scale"], case["q_len"], case["key_scale"], case["value_scale"])
         torch.testing.assert_close(out.double(), case["expected"], atol=2e-3, rtol=2 ** -8)
+
+
+def test_sink_term_closed_form():
+    # one query row, two keys: out = (e^{s0} v0 + e^{s1} v1) / (e^{s0} + e^{s1} + e^{sink})
+    q = torch.tensor([[[1.0, 0.0]]])                       # [q=1, Hq=1, D=2]
+    k = torch.tensor([[[2.0, 0.0]], [[-1.0, 0.0]]])        # [ctx=2, Hkv=1, D=2]
+    v = torch.tensor([[[1.0, 10.0]], [[3.0, -4.0]]])
+    sink = torch.tensor([[0.5]])
+    out = O.masked_attention(q, k, v, 1.0, torch.float32, True, None, sink)
+    e0, e1, es = math.exp(2.0), math.exp(-1.0), math.exp(0.5)
+    exp = torch.tensor([(e0 * 1.0 + e1 * 3.0) / (e0 + e1 + es), (e0 * 10.0 + e1 * -4.0) / (e0 + e1 + es)])
+    torch.testing.assert_close(out.view(-1), exp, atol=1e-6, rtol=1e-6)

@@ -143,6 +143,25 @@ def test_alibi(cuda):
     _check_stages(wl, res, 256, slopes)
 
 
+@pytest.mark.parametrize("ctx", [(300, 64, 1000), (100, 40, 250)])
+def test_attention_sinks(cuda, ctx):
+    import triton_op_amd as T
+
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(*ctx), q_len=2)
+    g = wl.to(cuda)
+    sinks = torch.linspace(-2.0, 3.0, wl.query.shape[1], dtype=torch.float32)
+    out = torch.full_like(g.query, float("nan"))
+    T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                             sinks=sinks.to(cuda))
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode_oracle(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                          wl.softmax_scale, 2, wl.key_scale, wl.value_scale, sinks=sinks)
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
+    plain = _oracle(wl)
+    assert float((plain.float() - ref.float()).abs().max()) > 5e-2  # the sinks do change the result
+
+
 def test_golden_fixtures(cuda):
     import glob
     import os

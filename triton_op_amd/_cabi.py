@@ -35,7 +35,7 @@ class PaDecodeArgs(C.Structure):
         [("struct_size", C.c_uint32), ("reserved0", C.c_int32)]
         + [(n, C.c_void_p) for n in (
             "output", "query", "key_cache", "value_cache", "context_lens", "block_tables", "q_lens",
-            "query_scale", "key_scale", "value_scale", "alibi_slopes", "exp_sums", "max_logits", "tmp_output",
+            "query_scale", "key_scale", "value_scale", "alibi_slopes", "sinks", "exp_sums", "max_logits", "tmp_output",
             "workspace")]
         + [(n, C.c_int32) for n in (
             "num_seqs", "num_kv_heads", "group_size", "q_len", "head_size", "block_size",

@@ -331,7 +331,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                         (int64_t)part * a.stride_tmp_p) * 2;
       char* op = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
-      const bool dir = ctx <= a.partition_size && a.output != nullptr;
+      const bool dir = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
       for (int r = row0 + kg; r < row0 + 16 * NT && r < Ge; r += 4) {
         if (li == 0) {
           a.max_logits[eo + r] = -INFINITY;
@@ -821,6 +821,20 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
     Pages pg_next = load_pages(part_start + kStepTokens);
     for (; sidx < n_fast; ++sidx) {
+      // Waves that share a SIMD do not progress evenly by themselves (the older one wins every
+      // arbitration and finishes a third earlier, leaving the SIMD half empty at the end): the further a
+      // wave is from its end, the higher its issue priority.
+      {
+        const int rem4 = (n_steps - sidx) * 4 / n_steps;
+        if (rem4 >= 3)
+          __builtin_amdgcn_s_setprio(3);
+        else if (rem4 == 2)
+          __builtin_amdgcn_s_setprio(2);
+        else if (rem4 == 1)
+          __builtin_amdgcn_s_setprio(1);
+        else
+          __builtin_amdgcn_s_setprio(0);
+      }
       const Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
       step.template operator()<true, true>(buf_a, tok0, pg_next);
       pg_next = pg_after;
@@ -846,7 +860,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                      (int64_t)part * a.stride_tmp_p) * 2;
   // a sequence that fits in one partition needs no merge: its partial is the result
-  const bool direct = ctx <= a.partition_size && a.output != nullptr;
+  const bool direct = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
   const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
   float l_tot[NT];
@@ -985,7 +999,7 @@ __global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
   uint32_t* out = reinterpret_cast<uint32_t*>((char*)a.output +
                                               ((int64_t)b * a.stride_out_s + (int64_t)(h * Ge + row) * a.stride_out_h) * 2) + lane;
   // SKIP_SINGLE: the partition kernel of the same call has written the rows of sequences with one partition
-  if (SKIP_SINGLE && n == 1) return;
+  if (SKIP_SINGLE && n == 1 && !a.sinks) return;
   if (n <= 0 || row >= qb * a.group_size) {
     *out = 0u;
     return;
@@ -1040,6 +1054,8 @@ __global__ __launch_bounds__(256) void pa_reduce_kernel(const PaDecodeArgs a) {
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) wsum += __shfl_xor(wsum, o);
+  // attention sink: one more term in the softmax denominator, exp(sink - M), with no value attached
+  if (a.sinks) wsum += __expf(a.sinks[h * Ge + row] - M_safe);
   const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
   *out = pack_bf16x2(acc0 * inv, acc1 * inv);
 }
@@ -1281,7 +1297,7 @@ int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
   int rc = pa_decode_partition(a, hip_stream);
   if (rc) return rc;
   // the partition kernel has written the rows of every sequence that fits in one partition itself
-  if (a->max_num_partitions == 1) return PA_OK;
+  if (a->max_num_partitions == 1 && !a->sinks) return PA_OK;
   return launch_reduce(a, hip_stream, true);
 }
 

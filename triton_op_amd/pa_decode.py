@@ -13,6 +13,9 @@ pa_decode_triton.py:523-685.  Differences, all additive:
 * `partition_size` may be any multiple of 256 (the reference's constant); by default the tuning
   layer picks it from the batch shape and the longest context;
 * `query_lens` gives a per-sequence number of new tokens (ragged MTP batches);
+* `sinks` gives an attention-sink logit per query row ([num_kv_heads * query_group_size], as the reference's
+  Gluon reduce kernel indexes it, pa_decode_triton_gluon_fp8.py:1118-1123): exp(sink - max) joins the softmax
+  denominator;
 * `workspace` is a zeroed int32 tensor of 64 bytes holding a work-item counter for ragged batches (one is
   allocated per call/plan when it is not given; calls that may overlap on the GPU need one each).
 
@@ -105,6 +108,7 @@ def plan_decode(
     partition_size: Optional[int] = None,
     query_lens: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
+    sinks: Optional[torch.Tensor] = None,
 ) -> DecodePlan:
     # ---- shapes (pa_decode_triton_gluon_fp8.py:1703-1722) ------------------------------------
     if output.dim() != 3:
@@ -221,6 +225,9 @@ def plan_decode(
     if alibi_slopes is not None:
         if alibi_slopes.dtype != torch.float32 or alibi_slopes.numel() != num_kv_heads * group or not alibi_slopes.is_contiguous():
             raise ValueError(f"alibi_slopes must be contiguous float32 [{num_kv_heads * group}]")
+    if sinks is not None:
+        if sinks.dtype != torch.float32 or sinks.numel() != rows_total or not sinks.is_contiguous() or sinks.device != dev:
+            raise ValueError(f"sinks must be contiguous float32 [{rows_total}] (one logit per query row) on {dev}")
     if query_lens is not None:
         if query_lens.dtype != torch.int32 or query_lens.numel() != num_seqs or not query_lens.is_contiguous():
             raise ValueError("query_lens must be contiguous int32 [num_seqs]")
@@ -277,6 +284,7 @@ def plan_decode(
     a.key_scale = _ptr(key_scale) if kv_mode != _cabi.PA_QUANT_NONE else None
     a.value_scale = _ptr(value_scale) if kv_mode != _cabi.PA_QUANT_NONE else None
     a.alibi_slopes = _ptr(alibi_slopes)
+    a.sinks = _ptr(sinks)
     a.exp_sums, a.max_logits, a.tmp_output = exp_sums.data_ptr(), max_logits.data_ptr(), tmp_output.data_ptr()
     # zeroed work-item counter for ragged batches; the kernels leave it zero, so the plan can be replayed
     if workspace is None:
@@ -301,7 +309,7 @@ def plan_decode(
     a.stride_tmp_s, a.stride_tmp_h, a.stride_tmp_p, a.stride_tmp_g = (tmp_output.stride(i) for i in range(4))
     a.stride_qscale_s, a.stride_kvscale_b, a.stride_kvscale_h = stride_qs, stride_kvs_b, stride_kvs_h
     keep = (output, query, key_cache, value_cache, sequence_lengths, block_tables, query_scale, key_scale,
-            value_scale, alibi_slopes, query_lens, workspace)
+            value_scale, alibi_slopes, query_lens, workspace, sinks)
     return DecodePlan(a, keep, exp_sums, max_logits, tmp_output, output)
 
 
@@ -328,6 +336,7 @@ def paged_attention_decode(
     partition_size: Optional[int] = None,
     query_lens: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
+    sinks: Optional[torch.Tensor] = None,
 ) -> Dict[str, object]:
     """Split-KV paged-attention decode; writes `output` in place on torch's current stream and
     returns the partition buffers under the reference's keys."""
@@ -335,7 +344,8 @@ def paged_attention_decode(
         output, query, key_cache, value_cache, sequence_lengths, block_tables, softmax_scale,
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
         num_sequence_partitions, alibi_slopes, exp_sums=exp_sums, max_logits=max_logits,
-        tmp_output=tmp_output, partition_size=partition_size, query_lens=query_lens, workspace=workspace)
+        tmp_output=tmp_output, partition_size=partition_size, query_lens=query_lens, workspace=workspace,
+        sinks=sinks)
     plan.run()
     return {
         "temporary_output": plan.tmp_output,
