@@ -151,6 +151,47 @@ int pa_decode_reduce(const PaDecodeArgs* args, void* hip_stream);
 int pa_decode(const PaDecodeArgs* args, void* hip_stream);
 
 /*
+ * KV-cache write: the step before the decode path.  Writes num_tokens new (key, value) rows
+ * [num_tokens, Hkv, D] (bf16) into the paged caches at slot_mapping[t] = block * block_size + offset
+ * (negative = skip), in the layouts the decode kernels read.  With an FP8 cache the rows are
+ * quantised on the way: per token and kv head (scale = amax / 448 written to the scale tensors), per
+ * tensor (the given scales are read), or cast as they are.  The reference has this step only as an
+ * offline whole-cache routine, quantize_kv_cache_symmetric (test_pa_mtp.py:294-369, over
+ * aiter.pertoken_quant), which pa_quantize_kv_cache below replaces directly.
+ */
+typedef struct PaKvWriteArgs {
+  uint32_t struct_size; /* = sizeof(PaKvWriteArgs) */
+  int32_t reserved0;
+  const void* key;             /* bf16 [num_tokens, Hkv, D] */
+  const void* value;           /* bf16 [num_tokens, Hkv, D] */
+  const int64_t* slot_mapping; /* [num_tokens] */
+  void* key_cache;             /* [blocks, Hkv, D/x, bs, x] */
+  void* value_cache;           /* [blocks, Hkv, D, bs] */
+  float* key_scale;            /* per token: [blocks, Hkv, bs, 1] written; per tensor: 1 value read */
+  float* value_scale;
+  int64_t num_tokens;
+  int32_t num_kv_heads;
+  int32_t head_size;           /* 128 */
+  int32_t block_size;
+  int32_t cache_dtype;         /* PA_DTYPE_* */
+  int32_t kv_quant_mode;       /* PA_QUANT_* */
+  int32_t reserved1;
+  int64_t stride_k_t, stride_k_h, stride_v_t, stride_v_h; /* elements; last dim contiguous */
+  int64_t stride_kc_b, stride_kc_h, stride_vc_b, stride_vc_h; /* cache block / head strides; inner dims dense */
+  int64_t stride_scale_b, stride_scale_h;
+} PaKvWriteArgs;
+
+int pa_kv_cache_write(const PaKvWriteArgs* args, void* hip_stream);
+
+/*
+ * Whole-cache per-token FP8 quantisation of a dense bf16 cache (x = 8) into a dense FP8 cache (x = 16)
+ * plus scales [num_blocks, Hkv, block_size, 1]: quantize_kv_cache_symmetric (test_pa_mtp.py:294-369).
+ */
+int pa_quantize_kv_cache(const void* key_cache_bf16, const void* value_cache_bf16, void* key_cache_fp8,
+                         void* value_cache_fp8, float* key_scale, float* value_scale, int64_t num_blocks,
+                         int32_t num_kv_heads, int32_t head_size, int32_t block_size, void* hip_stream);
+
+/*
  * Test hook: decodes n FP8 e4m3fn bytes (device pointer) to f32 (device pointer) with the same
  * conversion instructions the partition kernel uses, so the dequantisation table can be compared
  * with the format definition code by code.

@@ -40,6 +40,15 @@ def test_struct_layout_and_version(pa_lib):
             continue
         names += [n.strip().lstrip("*") for n in re.sub(r"^(const\s+)?[a-z0-9_]+\s*\**", "", decl, count=1).split(",")]
     assert names == [f[0] for f in _cabi.PaDecodeArgs._fields_]
+    body = re.search(r"typedef struct PaKvWriteArgs \{(.*?)\} PaKvWriteArgs;", _header(), re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if decl:
+            names += [n.strip().lstrip("*") for n in re.sub(r"^(const\s+)?[a-z0-9_]+\s*\**", "", decl, count=1).split(",")]
+    assert names == [f[0] for f in _cabi.PaKvWriteArgs._fields_]
+    assert C.sizeof(_cabi.PaKvWriteArgs) == 8 + 7 * 8 + 8 + 6 * 4 + 10 * 8
 
 
 def test_error_strings_and_null_arguments(pa_lib):

@@ -1,0 +1,94 @@
+"""The KV-cache write / quantise kernels against the torch formulas in kv_layout (same scale = amax/448,
+same float32 division, round to nearest even): the bytes and the scales must match exactly, and a cache
+written by the kernels must decode to the same attention output as one built on the host."""
+import pytest
+import torch
+
+from triton_op_amd import kv_layout as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("bs,nblk,h", [(16, 37, 2), (64, 5, 3), (1024, 2, 1)])
+def test_quantize_whole_cache_matches_torch_bit_for_bit(cuda, bs, nblk, h):
+    import triton_op_amd as T
+
+    g = torch.Generator().manual_seed(bs)
+    kc, vc = L.create_kv_cache(nblk, bs, h, 128, torch.bfloat16, generator=g, distribution="normal")
+    kc[1, 0, :, 3] = 0  # an all-zero key row: scale 1, bytes 0
+    kq_ref, ks_ref, vq_ref, vs_ref = L.quantize_kv_cache_per_token(kc, vc)
+    kq, ksf, vq, vsf, ks, vs = T.quantize_kv_cache_symmetric(kc.to(cuda), vc.to(cuda), torch.float8_e4m3fn)
+    torch.cuda.synchronize()
+    assert torch.equal(ks.cpu(), ks_ref) and torch.equal(vs.cpu(), vs_ref)
+    assert torch.equal(kq.cpu().view(torch.uint8), kq_ref.view(torch.uint8))
+    assert torch.equal(vq.cpu().view(torch.uint8), vq_ref.view(torch.uint8))
+    assert float(ks[1, 0, 3, 0]) == 1.0
+    assert ksf.shape == (h, nblk * bs) and torch.equal(ksf.cpu(), ks_ref.permute(1, 0, 2, 3).reshape(h, nblk * bs))
+    assert torch.equal(vsf.cpu(), vs_ref.permute(1, 0, 2, 3).reshape(h, nblk * bs))
+
+
+@pytest.mark.parametrize("mode", ["token", "tensor", "bf16"])
+def test_cache_write_then_decode(cuda, mode):
+    """Tokens appended through kv_cache_write (in two calls, scattered slots, one padding token) give the same
+    cache bytes as the host-side quantiser, and the decode op reads them back correctly."""
+    import triton_op_amd as T
+    from oracle import pa_oracle as O
+
+    bs, nblk, h, d = 16, 24, 2, 128
+    ctx = torch.tensor([70, 133], dtype=torch.int32)
+    g = torch.Generator().manual_seed(5)
+    perm = torch.randperm(nblk, generator=g).to(torch.int32)
+    bt = perm[:18].view(2, 9).contiguous()
+    toks = int(ctx.sum())
+    key = torch.randn(toks, h, d, generator=g).to(torch.bfloat16)
+    value = torch.randn(toks, h, d, generator=g).to(torch.bfloat16)
+    slots = torch.cat([bt[b].long().repeat_interleave(bs)[:int(ctx[b])] * bs + torch.arange(int(ctx[b])) % bs for b in range(2)])
+    # host reference cache
+    k_tok = torch.zeros(nblk, bs, h, d, dtype=torch.bfloat16)
+    v_tok = torch.zeros(nblk, bs, h, d, dtype=torch.bfloat16)
+    k_tok.view(-1, h, d)[slots] = key
+    v_tok.view(-1, h, d)[slots] = value
+    kc16, vc16 = L.tokens_to_key_cache(k_tok), L.tokens_to_value_cache(v_tok)
+    dev = cuda
+    if mode == "bf16":
+        kc = torch.zeros_like(kc16, device=dev)
+        vc = torch.zeros_like(vc16, device=dev)
+        ks = vs = None
+        kref, vref, ksr, vsr = kc16, vc16, None, None
+    else:
+        kc = torch.zeros(nblk, h, d // 16, bs, 16, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        vc = torch.zeros(nblk, h, d, bs, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        if mode == "token":
+            kref, ksr, vref, vsr = L.quantize_kv_cache_per_token(kc16, vc16)
+            ks = torch.ones(nblk, h, bs, 1, device=dev)
+            vs = torch.ones(nblk, h, bs, 1, device=dev)
+        else:
+            ksr = (key.float().abs().max() / 448.0).to(torch.float32)
+            vsr = (value.float().abs().max() / 448.0).to(torch.float32)
+            kref = L.tokens_to_key_cache((k_tok.float() / ksr).to(torch.float8_e4m3fn))
+            vref = L.tokens_to_value_cache((v_tok.float() / vsr).to(torch.float8_e4m3fn))
+            ks, vs = ksr.to(dev), vsr.to(dev)
+    # append in two calls; the second carries a padding token (slot -1)
+    cut = 90
+    T.kv_cache_write(key[:cut].to(dev), value[:cut].to(dev), kc, vc, slots[:cut].to(dev), ks, vs)
+    k2 = torch.cat([key[cut:], key[:1]]).to(dev)
+    v2 = torch.cat([value[cut:], value[:1]]).to(dev)
+    s2 = torch.cat([slots[cut:], torch.tensor([-1])]).to(dev)
+    T.kv_cache_write(k2, v2, kc, vc, s2, ks, vs)
+    torch.cuda.synchronize()
+    view = torch.uint8 if mode != "bf16" else torch.int16
+    assert torch.equal(kc.cpu().view(view), kref.view(view))
+    assert torch.equal(vc.cpu().view(view), vref.view(view))
+    if mode == "token":
+        live = torch.zeros(nblk * bs, dtype=torch.bool)
+        live[slots] = True
+        live = live.view(nblk, 1, bs, 1).expand(nblk, h, bs, 1)
+        assert torch.equal(ks.cpu()[live], ksr[live]) and torch.equal(vs.cpu()[live], vsr[live])
+        assert bool((ks.cpu()[~live] == 1).all())  # untouched
+    # decode from the cache the kernels wrote
+    q = torch.randn(2, 16, d, generator=g).to(torch.bfloat16)
+    out = torch.empty(2, 16, d, dtype=torch.bfloat16, device=dev)
+    T.paged_attention_decode(out, q.to(dev), kc, vc, ctx.to(dev), bt.to(dev), d ** -0.5, 1, 133, torch.bfloat16, None, ks, vs)
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode_oracle(q, kref, vref, ctx, bt, d ** -0.5, 1, ksr, vsr)
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=2e-2, rtol=2e-2)

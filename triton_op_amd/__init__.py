@@ -7,6 +7,8 @@ from .pa_decode import (  # noqa: F401
     plan_decode,
     select_partition_size,
 )
+from .kv_cache import kv_cache_write, quantize_kv_cache_symmetric  # noqa: F401
 from . import kv_layout, workloads  # noqa: F401
 
-__all__ = ["paged_attention_decode", "plan_decode", "DecodePlan", "select_partition_size", "kv_layout", "workloads"]
+__all__ = ["paged_attention_decode", "plan_decode", "DecodePlan", "select_partition_size", "kv_cache_write",
+           "quantize_kv_cache_symmetric", "kv_layout", "workloads"]

@@ -27,6 +27,8 @@ EXPORTED_SYMBOLS = (
     "pa_decode_reduce",
     "pa_decode",
     "pa_debug_fp8_decode",
+    "pa_kv_cache_write",
+    "pa_quantize_kv_cache",
 )
 
 
@@ -48,6 +50,18 @@ class PaDecodeArgs(C.Structure):
             "stride_bt_s", "stride_es_s", "stride_es_h", "stride_es_p",
             "stride_tmp_s", "stride_tmp_h", "stride_tmp_p", "stride_tmp_g",
             "stride_qscale_s", "stride_kvscale_b", "stride_kvscale_h")]
+    )
+
+
+class PaKvWriteArgs(C.Structure):
+    _fields_ = (
+        [("struct_size", C.c_uint32), ("reserved0", C.c_int32)]
+        + [(n, C.c_void_p) for n in ("key", "value", "slot_mapping", "key_cache", "value_cache", "key_scale", "value_scale")]
+        + [("num_tokens", C.c_int64)]
+        + [(n, C.c_int32) for n in ("num_kv_heads", "head_size", "block_size", "cache_dtype", "kv_quant_mode", "reserved1")]
+        + [(n, C.c_int64) for n in (
+            "stride_k_t", "stride_k_h", "stride_v_t", "stride_v_h", "stride_kc_b", "stride_kc_h", "stride_vc_b",
+            "stride_vc_h", "stride_scale_b", "stride_scale_h")]
     )
 
 
@@ -85,6 +99,10 @@ def load_library(path: str = None) -> C.CDLL:
             fn.argtypes = [C.POINTER(PaDecodeArgs), C.c_void_p]
         lib.pa_debug_fp8_decode.restype = C.c_int
         lib.pa_debug_fp8_decode.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
+        lib.pa_kv_cache_write.restype = C.c_int
+        lib.pa_kv_cache_write.argtypes = [C.POINTER(PaKvWriteArgs), C.c_void_p]
+        lib.pa_quantize_kv_cache.restype = C.c_int
+        lib.pa_quantize_kv_cache.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
         if lib.pa_decode_abi_version() != PA_DECODE_ABI_VERSION:
             raise PaDecodeLibraryError("libpa_decode.so has a different ABI version; rebuild it")
         if lib.pa_decode_args_size() != C.sizeof(PaDecodeArgs):

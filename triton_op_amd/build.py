@@ -13,7 +13,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = [os.path.join(HERE, "csrc", "pa_decode.hip")]
+SOURCES = [os.path.join(HERE, "csrc", "pa_decode.hip"), os.path.join(HERE, "csrc", "pa_kv_cache.hip")]
 HEADERS = [os.path.join(HERE, "..", "include", "pa_decode.h")]
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
