@@ -1,36 +1,36 @@
 // Split-KV paged-attention decode for MI355X (gfx950 / CDNA4): partition kernel, reduce kernel
 // and the C ABI declared in include/pa_decode.h.
 //
-// Work decomposition.  One wavefront (64 lanes) owns one (sequence, kv head, partition) and keeps
-// private online-softmax state (m, l, O); nothing is shared between waves, so there are no
-// workgroup barriers.  A partition is walked in steps of 64 tokens (four 16-token tiles):
+// Work decomposition.  A workgroup of 1, 2 or 4 waves owns one item: (sequence, partition, 16-row
+// query tile, kv head).  Each wave streams a contiguous slice of the partition in steps of 64 tokens
+// (four 16-token tiles) with private online-softmax state (m, l, O); the waves merge through LDS at the
+// end.  A sequence that fits in one partition gets its final output from this kernel directly.
 //
 //   K tile  (16 tokens x 128 dims): every lane loads 16 bytes = one [token][16-byte chunk] cell of
 //           the cache; lanes 0-15 are the 16 tokens of a page, lane>>4 picks the chunk row, so a
-//           wave load covers 4 x 256 contiguous bytes in storage order.  The 16 bytes are the A
-//           operand of two 16x16x32 MFMA k-steps (the dot product does not care in which order the
-//           head dimension is summed, so the query operand is loaded in the matching order).
-//   S^T = K Q^T on v_mfma_f32_16x16x32_bf16: tokens are the M rows, query rows (GQA group x MTP
-//           position, padded to 16) are the N columns, so a lane ends up with 4 tokens of ONE
-//           query row and the softmax max/sum need only two cross-lane steps (lane^16, lane^32).
-//   P       goes through a wave-private LDS tile to become the B operand of the second MFMA.
+//           wave load covers 4 x 256 contiguous bytes in storage order.  The dot product does not care
+//           in which order the head dimension is summed, so the query operand is built in the order
+//           the loads deliver it.
+//   S^T = K Q^T: tokens are the M rows, query rows (GQA group x MTP position, padded to 16) are
+//           the N columns, so a lane ends up with 4 tokens of ONE query row per tile and the softmax
+//           max/sum need only two cross-lane steps (lane^16, lane^32).
 //   V tile  (128 dims x 16 tokens): every lane loads 16 bytes = 16 tokens of one head dim, lanes
-//           0-15 are 16 consecutive dims (256 contiguous bytes), lane>>4 picks one of the four
-//           tiles of the step.  O^T = V^T P^T accumulates in 8 MFMA tiles of [16 dims x 16 rows].
+//           0-15 are 16 consecutive dims (256 contiguous bytes with block 16), lane>>4 picks one of
+//           the four tiles of the step.  O^T = V^T P^T accumulates in 8 MFMA tiles of [16 dims x 16 rows].
 //
-// FP8 e4m3fn is widened to bf16 exactly (3 mantissa bits fit in 7); per-tensor scales are folded
-// into the softmax scale (K) and the epilogue (V), per-token scales multiply S and P in f32.
-// The next step's K/V/page ids are in flight while the current step is computed.
+// FP8 cache: the cache bytes are MFMA operands as they are (v_mfma_f32_16x16x128_f8f6f4 for Q K^T,
+// v_mfma_f32_16x16x32_fp8_fp8 for P V); the bf16 query and P are each carried as an FP8 head plus an
+// FP8 residual (x*c = hi + lo, every product exact in the f32 accumulator), about 2^-8 relative per
+// element, so there is no FP8->bf16 conversion work at all; P reaches the B-operand layout through a 4x4
+// (lane group x register) transpose with v_permlane{16,32}_swap, not through LDS.  Per-tensor scales
+// fold into the softmax scale (K) and the epilogue (V); per-token scales multiply S and P in f32.
+// bf16 cache: bf16 MFMA (v_mfma_f32_16x16x32_bf16), P through a wave-private LDS tile.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
 
 #include "../../include/pa_decode.h"
-
-#ifndef PA_CVT_SCALEF32
-#define PA_CVT_SCALEF32 0
-#endif
 
 namespace {
 
@@ -44,7 +44,6 @@ typedef __attribute__((ext_vector_type(8))) int i32x8;
 
 constexpr int kHeadSize = 128;
 constexpr int kStepTokens = 64;     // tokens per pipeline step (4 tiles of 16)
-constexpr int kChunkTokens = 256;   // page ids are fetched for 256 tokens (4 steps) at a time
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kPRowBytes = 144;     // 64 tokens * 2 B + 16 B pad per query row of the P tile
 
@@ -56,20 +55,10 @@ union Bf16x8Bits {
 
 // two FP8 e4m3fn bytes -> two bf16, exactly (an e4m3 value has 3 mantissa bits, bf16 keeps 7)
 __device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t word, bool high_half) {
-#if PA_CVT_SCALEF32
-  union {
-    bf16x2 v;
-    uint32_t u;
-  } r;
-  r.v = high_half ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)word, 1.0f, true)
-                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)word, 1.0f, false);
-  return r.u;
-#else
   // v_cvt_pk_f32_fp8, then keep the upper 16 bits of each f32
   f32x2 f = high_half ? __builtin_amdgcn_cvt_pk_f32_fp8((int)word, true)
                       : __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
   return __builtin_amdgcn_perm(__float_as_uint(f[1]), __float_as_uint(f[0]), 0x07060302u);
-#endif
 }
 
 __device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t lo, uint32_t hi) {
@@ -203,18 +192,13 @@ struct StepData {
 //
 // BS16 (block size 16) turns every stride inside a page into a compile-time constant, so the loads
 // of a tile share one address register pair and differ by immediate offsets.
-// FP8MATH (FP8 cache only) feeds the cache bytes to the FP8 MFMAs as they are: Q and P are split into
-// an FP8 head and an FP8 residual (q*c = hi + lo, each product exact in the f32 accumulator), which
-// keeps them at bf16-like precision, costs two MFMAs where the bf16 path has one, and removes every
-// FP8->bf16 conversion and the LDS round trip of P (a 4x4 lane-group transpose with
-// v_permlane{16,32}_swap puts P into the B-operand layout).
 constexpr int kQueueMaxSeqs = 2048;  // sequences the item table of the queued launch can hold
 
-template <int NT, int KVT, bool PER_TOKEN, bool FP8MATH, bool BS16, int WAVES, int OCC, int DEPTH, bool QUEUE>
+template <int NT, int KVT, bool PER_TOKEN, bool BS16, int WAVES, int OCC, bool QUEUE>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_kernel(const PaDecodeArgs a) {
   constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
-  static_assert(kFp8 || !FP8MATH, "FP8 MFMA path needs an FP8 cache");
+  constexpr bool FP8MATH = kFp8;  // an FP8 cache is multiplied on the FP8 MFMAs, a bf16 cache on the bf16 ones
   constexpr int esz = kFp8 ? 1 : 2;
   typedef StepData<KVT, PER_TOKEN> SD;
 
@@ -422,18 +406,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 
   // ---- first loads go out before anything else is set up ---------------------------------------------
   const int n_steps = (part_end - part_start + kStepTokens - 1) / kStepTokens;
-  // DEPTH 2: steps alternate between two buffers, each refilled in place for the step after next;
-  // DEPTH 1: one buffer, refilled in place for the next step
-  SD buf_a, buf_b;
+  SD buf_a;  // one step of cache data, refilled in place for the next step
   if (active) {
     Pages pg0 = load_pages(part_start);
     issue_k(buf_a, pg0);
     issue_v(buf_a, pg0);
-    if (DEPTH == 2 && n_steps > 1) {
-      Pages pg1 = load_pages(part_start + kStepTokens);
-      issue_k(buf_b, pg1);
-      issue_v(buf_b, pg1);
-    }
   }
 
   // ---- per-lane row bookkeeping -------------------------------------------------------------------------
@@ -566,21 +543,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       } else
 #pragma unroll
       for (int ld = 0; ld < SD::NKL; ++ld) {
-        if constexpr (kFp8) {
-          bf16x8 a0 = fp8x8_to_bf16x8(sd.k[j][ld][0], sd.k[j][ld][1]);
-          bf16x8 a1 = fp8x8_to_bf16x8(sd.k[j][ld][2], sd.k[j][ld][3]);
+        Bf16x8Bits ka;
+        ka.u = sd.k[j][ld];
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[nt][2 * ld], s[nt][j], 0, 0, 0);
-            s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[nt][2 * ld + 1], s[nt][j], 0, 0, 0);
-          }
-        } else {
-          Bf16x8Bits ka;
-          ka.u = sd.k[j][ld];
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka.v, qreg[nt][ld], s[nt][j], 0, 0, 0);
-        }
+        for (int nt = 0; nt < NT; ++nt)
+          s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka.v, qreg[nt][ld], s[nt][j], 0, 0, 0);
       }
     }
     f32x4 ks_cur[PER_TOKEN ? 4 : 1];
@@ -756,17 +723,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       }
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
-        bf16x8 va;
-        if constexpr (kFp8) {
-          va = fp8x8_to_bf16x8(sd.v[db][0][2 * hf], sd.v[db][0][2 * hf + 1]);
-        } else {
-          Bf16x8Bits t;
-          t.u = sd.v[db][hf];
-          va = t.v;
-        }
+        Bf16x8Bits va;
+        va.u = sd.v[db][hf];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-          acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[nt], acc[nt][db], 0, 0, 0);
+          acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb[nt], acc[nt][db], 0, 0, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -782,42 +743,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   n_full = n_full < 0 ? 0 : n_full;
   int sidx = 0;
   int tok0 = part_start;
-  if (!active) {
-    // nothing to stream
-  } else if constexpr (DEPTH == 2) {
-    // pairs of unmasked steps that both have a step two ahead to request
-    const int n_pf = n_steps - 2;
-    const int n_fast = (n_full < n_pf ? n_full : n_pf) & ~1;
-    Pages pg_a = load_pages(part_start + 2 * kStepTokens);  // pages of the step buf_a is refilled for
-    Pages pg_b = load_pages(part_start + 3 * kStepTokens);
-    for (; sidx < n_fast; sidx += 2) {
-      const Pages na = load_pages(tok0 + 4 * kStepTokens);
-      step.template operator()<true, true>(buf_a, tok0, pg_a);
-      const Pages nb = load_pages(tok0 + 5 * kStepTokens);
-      step.template operator()<true, true>(buf_b, tok0 + kStepTokens, pg_b);
-      pg_a = na;
-      pg_b = nb;
-      tok0 += 2 * kStepTokens;
-    }
-    // the two steps already requested, then (ALiBi, or an odd step left over) load-and-compute
-    if (n_full >= n_steps) {
-      step.template operator()<true, false>(buf_a, tok0, pg_a);
-      if (sidx + 1 < n_steps) step.template operator()<true, false>(buf_b, tok0 + kStepTokens, pg_b);
-      sidx += 2;
-    } else {
-      step.template operator()<false, false>(buf_a, tok0, pg_a);
-      if (sidx + 1 < n_steps) step.template operator()<false, false>(buf_b, tok0 + kStepTokens, pg_b);
-      sidx += 2;
-      tok0 += 2 * kStepTokens;
-      for (; sidx < n_steps; ++sidx) {
-        const Pages pg = load_pages(tok0);
-        issue_k(buf_a, pg);
-        issue_v(buf_a, pg);
-        step.template operator()<false, false>(buf_a, tok0, pg);
-        tok0 += kStepTokens;
-      }
-    }
-  } else {
+  if (active) {
     const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
     Pages pg_next = load_pages(part_start + kStepTokens);
     for (; sidx < n_fast; ++sidx) {
@@ -1109,10 +1035,9 @@ bool use_queue(const PaDecodeArgs& a) {
   return !off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr;
 }
 
-template <int NT, int KVT, bool PT, bool FP8MATH, bool BS16, int W>
+template <int NT, int KVT, bool PT, bool BS16, int W>
 int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   constexpr int OCC = NT == 1 ? 2 : 1;
-  constexpr int DEPTH = 1;
   const int ge = a.q_len * a.group_size;
   const int row_tiles = (ge + 16 * NT - 1) / (16 * NT);
   const long long blocks = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * row_tiles;
@@ -1120,10 +1045,10 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   if (use_queue(a)) {
     long long resident = (long long)device_num_cus() * 4 * OCC / W;
     resident = resident < blocks ? resident : blocks;
-    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, FP8MATH, BS16, W, OCC, DEPTH, true>), dim3((unsigned)resident),
+    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)resident),
                        dim3(64 * W), 0, stream, a);
   } else
-  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, FP8MATH, BS16, W, OCC, DEPTH, false>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
+  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
@@ -1160,17 +1085,17 @@ int waves_per_workgroup(const PaDecodeArgs& a, int nt) {
   return w >= 4 ? 4 : (w >= 2 ? 2 : 1);
 }
 
-template <int KVT, bool PT, bool FP8MATH, bool BS16>
+template <int KVT, bool PT, bool BS16>
 int launch_partition_nt(const PaDecodeArgs& a, int nt, hipStream_t stream) {
   const int w = waves_per_workgroup(a, nt);
   switch (nt) {
     case 1:
-      if (w == 4) return launch_partition_w<1, KVT, PT, FP8MATH, BS16, 4>(a, stream);
-      if (w == 2) return launch_partition_w<1, KVT, PT, FP8MATH, BS16, 2>(a, stream);
-      return launch_partition_w<1, KVT, PT, FP8MATH, BS16, 1>(a, stream);
+      if (w == 4) return launch_partition_w<1, KVT, PT, BS16, 4>(a, stream);
+      if (w == 2) return launch_partition_w<1, KVT, PT, BS16, 2>(a, stream);
+      return launch_partition_w<1, KVT, PT, BS16, 1>(a, stream);
     case 2:
-      if (w == 2) return launch_partition_w<2, KVT, PT, FP8MATH, BS16, 2>(a, stream);
-      return launch_partition_w<2, KVT, PT, FP8MATH, BS16, 1>(a, stream);
+      if (w == 2) return launch_partition_w<2, KVT, PT, BS16, 2>(a, stream);
+      return launch_partition_w<2, KVT, PT, BS16, 1>(a, stream);
   }
   return PA_ERR_UNSUPPORTED;
 }
@@ -1281,13 +1206,13 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
     const bool bs16 = a->block_size == 16 && a->stride_k_c == 256 &&
                       (a->v_transposed ? a->stride_v_2 == 2048 : a->stride_v_2 == 16);
     if (bs16)
-      return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true, true>(*a, nt, stream)
-                : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true, true>(*a, nt, stream);
-    return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true, false>(*a, nt, stream)
-              : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true, false>(*a, nt, stream);
+      return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true>(*a, nt, stream)
+                : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true>(*a, nt, stream);
+    return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, false>(*a, nt, stream)
+              : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, false>(*a, nt, stream);
   }
   if (pt) return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
-  return launch_partition_nt<PA_DTYPE_BF16, false, false, false>(*a, nt, stream);
+  return launch_partition_nt<PA_DTYPE_BF16, false, false>(*a, nt, stream);
 }
 
 int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) { return launch_reduce(a, hip_stream, false); }
