@@ -114,6 +114,16 @@ CASES = {
                             transposed_v=True),
     "fp8_transV_bs1024": dict(batch=2, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(1500, 3000),
                               block_size=1024, transposed_v=True),
+    # more than 16 query rows per kv head over an FP8 cache: the row tiles share one pass over the pages
+    "fp8_bs64_g16_q2": dict(batch=3, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(1500, 63, 300), block_size=64,
+                            q_len=2),
+    "fp8_token_bs1024_g8_q4": dict(batch=3, num_q_heads=8, num_kv_heads=1, context_lens=_ctx(1500, 1024, 3000),
+                                   block_size=1024, q_len=4, scale_mode="token"),
+    "fp8_transV_bs16_g16_q3": dict(batch=3, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(300, 64, 1000),
+                                   transposed_v=True, q_len=3),
+    "fp8_token_transV_bs64_g8_q3": dict(batch=2, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(1500, 200),
+                                        block_size=64, transposed_v=True, q_len=3, scale_mode="token"),
+    "fp8_g8_q4_long": dict(batch=2, num_q_heads=8, num_kv_heads=1, context_lens=_ctx(9000, 4097), q_len=4),
     "bf16_transV_bs64": dict(batch=2, num_q_heads=8, num_kv_heads=2, context_lens=_ctx(150, 300), block_size=64,
                              kv_dtype="bf16", scale_mode="none", transposed_v=True),
 }
@@ -135,28 +145,30 @@ def test_parity_stagewise_and_end_to_end(cuda, name, partition_size):
     assert thr < 1e-2, thr
 
 
-def test_alibi(cuda):
-    wl = _make(**CASES["fp8_g8"])
+@pytest.mark.parametrize("name", ["fp8_g8", "fp8_g10_q3", "fp8_token_g16_q4"])
+def test_alibi(cuda, name):
+    wl = _make(**CASES[name])
     slopes = torch.linspace(0.01, 0.3, wl.num_q_heads, dtype=torch.float32)
     out, res = _run(wl, cuda, alibi=slopes)
     torch.testing.assert_close(out.float(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
     _check_stages(wl, res, 256, slopes)
 
 
+@pytest.mark.parametrize("q_len", [2, 4])
 @pytest.mark.parametrize("ctx", [(300, 64, 1000), (100, 40, 250)])
-def test_attention_sinks(cuda, ctx):
+def test_attention_sinks(cuda, ctx, q_len):
     import triton_op_amd as T
 
-    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(*ctx), q_len=2)
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(*ctx), q_len=q_len)
     g = wl.to(cuda)
     sinks = torch.linspace(-2.0, 3.0, wl.query.shape[1], dtype=torch.float32)
     out = torch.full_like(g.query, float("nan"))
     T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
-                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
-                             sinks=sinks.to(cuda))
+                             g.softmax_scale, q_len, g.max_context_len, torch.bfloat16, None, g.key_scale,
+                             g.value_scale, sinks=sinks.to(cuda))
     torch.cuda.synchronize()
     ref = O.paged_attention_decode_oracle(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
-                                          wl.softmax_scale, 2, wl.key_scale, wl.value_scale, sinks=sinks)
+                                          wl.softmax_scale, q_len, wl.key_scale, wl.value_scale, sinks=sinks)
     torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
     plain = _oracle(wl)
     assert float((plain.float() - ref.float()).abs().max()) > 5e-2  # the sinks do change the result
@@ -184,10 +196,12 @@ def test_golden_fixtures(cuda):
         assert err < 6e-3, (f, err)
 
 
-def test_stale_cache_contents_are_never_used(cuda):
+@pytest.mark.parametrize("q_len", [2, 4])
+def test_stale_cache_contents_are_never_used(cuda, q_len):
     """Slots past context_len in the last page, pages named by unused block-table entries, and their
     per-token scales, hold NaN bytes: the result must not change (and must not be NaN)."""
-    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(5, 250, 1001), scale_mode="token", q_len=2)
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(5, 250, 1001), scale_mode="token",
+               q_len=q_len)
     ref_out, _ = _run(wl, cuda)
     kc, vc = wl.key_cache.clone().view(torch.uint8), wl.value_cache.clone().view(torch.uint8)
     ks, vs = wl.key_scale.clone(), wl.value_scale.clone()
@@ -215,8 +229,9 @@ def test_stale_cache_contents_are_never_used(cuda):
     assert torch.equal(out.view(torch.int16), ref_out.view(torch.int16))
 
 
-def test_block_permutation_invariance_bit_exact(cuda):
-    wl = _make(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(700, 64, 2049, 300), q_len=2)
+@pytest.mark.parametrize("q_len", [2, 3])
+def test_block_permutation_invariance_bit_exact(cuda, q_len):
+    wl = _make(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(700, 64, 2049, 300), q_len=q_len)
     base, _ = _run(wl, cuda)
     n = wl.key_cache.shape[0]
     perm = torch.randperm(n, generator=torch.Generator().manual_seed(3))
@@ -252,32 +267,44 @@ def test_caller_buffers_strided_inputs_and_twin_entry_point(cuda):
     assert (es[1, :, 1:] == 7.0).all() and (to[1, :, 1:] == 7.0).all()
 
 
-def test_fp8_query_with_scales(cuda):
+@pytest.mark.parametrize("q_len", [2, 4])
+def test_fp8_query_with_scales(cuda, q_len):
     """FP8 query with a per-row scale, the reference Gluon entry point's own contract
     (pa_decode_triton_gluon_fp8.py:747-755,889-903)."""
     import triton_op_amd as T
     from triton_op_amd import kv_layout as L
 
-    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000), q_len=2, scale_mode="token")
+    wl = _make(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000), q_len=q_len,
+               scale_mode="token")
     qq, qs = L.pertoken_quant(wl.query.float())
     g = wl.to(cuda)
     out = torch.empty_like(g.query)
     T.paged_attention_decode(out, qq.to(cuda), g.key_cache, g.value_cache, g.context_lens, g.block_tables,
-                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, qs.to(cuda), g.key_scale,
+                             g.softmax_scale, q_len, g.max_context_len, torch.bfloat16, qs.to(cuda), g.key_scale,
                              g.value_scale)
     torch.cuda.synchronize()
     ref = O.paged_attention_decode_oracle(qq, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
-                                          wl.softmax_scale, 2, wl.key_scale, wl.value_scale, query_scale=qs)
+                                          wl.softmax_scale, q_len, wl.key_scale, wl.value_scale, query_scale=qs)
     torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
     qs0 = torch.tensor(float(wl.query.float().abs().max()) / 448.0)
     qq0 = (wl.query.float() / qs0).to(torch.float8_e4m3fn)
     T.paged_attention_decode(out, qq0.to(cuda), g.key_cache, g.value_cache, g.context_lens, g.block_tables,
-                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, qs0.to(cuda), g.key_scale,
+                             g.softmax_scale, q_len, g.max_context_len, torch.bfloat16, qs0.to(cuda), g.key_scale,
                              g.value_scale)
     torch.cuda.synchronize()
     ref0 = O.paged_attention_decode_oracle(qq0, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
-                                           wl.softmax_scale, 2, wl.key_scale, wl.value_scale, query_scale=qs0)
+                                           wl.softmax_scale, q_len, wl.key_scale, wl.value_scale, query_scale=qs0)
     torch.testing.assert_close(out.float().cpu(), ref0.float(), atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("name", ["fp8_g8", "fp8_token_g16_q4"])
+def test_negative_softmax_scale(cuda, name):
+    """A negative scale turns the row maximum of the raw logits into the minimum of the scaled ones: the
+    kernels must not assume the scale's sign when they take maxima before scaling."""
+    wl = _make(**CASES[name])
+    wl = type(wl)(**{**wl.__dict__, "softmax_scale": -wl.softmax_scale})
+    out, _ = _run(wl, cuda, partition_size=512)
+    torch.testing.assert_close(out.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
 def test_c_abi_rejects_bad_arguments(cuda, pa_lib):

@@ -1219,8 +1219,10 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     l_run = l_run * alpha + psum * inv_pmul;
     // the accumulator is rescaled only when some row's maximum (or the V scale unit) moved
     const float alpha_acc = alpha * vfac;
+    if (__builtin_amdgcn_ballot_w64(alpha_acc != 1.f)) {
 #pragma unroll
-    for (int db = 0; db < 8; ++db) acc[db] *= alpha_acc;
+      for (int db = 0; db < 8; ++db) acc[db] *= alpha_acc;
+    }
 
     // lane group kg holds, per tile j, tokens 4kg..4kg+3; the B operand of O^T += V^T P^T wants lane group
     // kg to hold all 16 tokens of tile kg: a 4x4 transpose over (lane group, register)
@@ -1532,7 +1534,12 @@ template <bool PT, bool BS16>
 int launch_partition_shared(const PaDecodeArgs& a, hipStream_t stream) {
   const long long blocks = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL((pa_partition_shared_kernel<PT, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  // ring depth / waves per SIMD: without per-token scales the kernel fits 128 registers, and a fourth workgroup
+  // per CU is worth more than a deeper ring (measured); with them it needs about 140
+  if constexpr (PT)
+    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else
+    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
@@ -1611,6 +1618,19 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   // up to 4 waves (at least 256 tokens each); no wave is given more than 2048 tokens, which keeps ragged
   // batches balanced.
   const int total_tiles = (rows_per_group + 15) / 16;
+  if (use_shared_stream(PA_DTYPE_FP8_E4M3FN, rows_per_group)) {
+    // All row tiles of a kv head in one workgroup that walks its partition alone: three workgroups fit a CU, and
+    // no workgroup gets more than 4096 tokens (measured on a ragged batch: 3072-4096 is the flat optimum, 8192
+    // costs 7 % in balance, 1024 costs 8 % in partials and merge).
+    const long long slots = (long long)num_cus * 3;
+    const long long items = (long long)num_seqs * num_kv_heads;
+    for (int parts = 1;; ++parts) {
+      int ps = (max_context_len + parts - 1) / parts;
+      ps = (ps + 255) / 256 * 256;
+      if (ps <= 256) return 256;
+      if (ps <= 4096 && items * parts >= slots) return ps;
+    }
+  }
   const int nt = tiles_per_workgroup(total_tiles);
   const int cap_w = nt <= 1 ? 4 : 2;
   const long long slots = (long long)num_cus * 4 * (nt <= 1 ? 2 : 1);
