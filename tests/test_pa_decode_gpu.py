@@ -297,6 +297,30 @@ def test_fp8_query_with_scales(cuda, q_len):
     torch.testing.assert_close(out.float().cpu(), ref0.float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("with_sinks", [False, True])
+def test_many_rows_take_the_four_rows_per_wave_reduce(cuda, with_sinks):
+    """16384 output rows and more are merged four rows per wave: up to 8 partitions through the all-loads-first
+    path, more through the row loop; padding rows of a ragged batch and single-partition sequences are mixed in."""
+    import triton_op_amd as T
+
+    gen = torch.Generator().manual_seed(11)
+    ctx = torch.randint(1, 1200, (128,), generator=gen, dtype=torch.int32)
+    ctx[:6] = torch.tensor([3000, 2049, 256, 257, 1, 2900], dtype=torch.int32)
+    ql = torch.randint(1, 3, (128,), generator=gen, dtype=torch.int32)
+    wl = _make(batch=128, num_q_heads=64, num_kv_heads=8, context_lens=torch.maximum(ctx, ql), q_len=2, q_lens=ql)
+    g = wl.to(cuda)
+    sinks = torch.linspace(-2.0, 3.0, wl.query.shape[1], dtype=torch.float32) if with_sinks else None
+    out = torch.full_like(g.query, float("nan"))
+    T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                             g.softmax_scale, 2, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                             partition_size=256, query_lens=g.q_lens, sinks=None if sinks is None else sinks.to(cuda))
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode_oracle(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                          wl.softmax_scale, wl.q_lens, wl.key_scale, wl.value_scale, sinks=sinks)
+    assert not torch.isnan(out.float()).any()
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
+
+
 @pytest.mark.parametrize("name", ["fp8_g8", "fp8_token_g16_q4"])
 def test_negative_softmax_scale(cuda, name):
     """A negative scale turns the row maximum of the raw logits into the minimum of the scaled ones: the
