@@ -561,7 +561,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 
     // FP8 math, per-token V scales: P carries v_scale / v_run (<= 1); the accumulator is kept in units
     // of the running maximum v_run
-    float vfac = 1.f, pmul = 256.f;
+    // FP8 math: P is produced already multiplied by pmul = 256 / v_run; log2(pmul) rides in the exponent's
+    // additive term, so the factor costs nothing per element
+    float vfac = 1.f, log2_pmul = FP8MATH ? 8.f : 0.f, inv_pmul = FP8MATH ? 1.f / 256.f : 1.f;
     f32x4 vs_cur[(PER_TOKEN && FP8MATH) ? 4 : 1];
     if constexpr (PER_TOKEN && FP8MATH) {
       float vmx = 0.f;
@@ -579,8 +581,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       }
       vmx = quad_row_max(vmx);
       const float v_new = fmaxf(v_run, vmx);
-      vfac = v_run / v_new;
-      pmul = 256.f / v_new;
+      vfac = v_new == v_run ? 1.f : v_run * __builtin_amdgcn_rcpf(v_new);
+      log2_pmul = 8.f - __builtin_amdgcn_logf(v_new);
+      inv_pmul = v_new * (1.f / 256.f);
       v_run = v_new;
     }
     uint32_t ph[FP8MATH ? NT : 1][4], pl[FP8MATH ? NT : 1][4];  // FP8 math: P head / residual, 4 tokens per dword
@@ -593,11 +596,12 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float v = s[nt][j][r] * rs;
+          // FULL: the row's scale (>= 0 on this path) is applied inside the exponent's fma, and to the maximum once
+          float v = s[nt][j][r];
           if constexpr (PER_TOKEN) v *= ks_cur[j][r];
           if constexpr (!FULL) {
             const int col = tok0 + 16 * j + 4 * kg + r;
-            v += slope2[nt] * (float)(col - ctx + 1);
+            v = v * rs + slope2[nt] * (float)(col - ctx + 1);
             v = col < limit[nt] ? v : -INFINITY;
           }
           s[nt][j][r] = v;
@@ -605,17 +609,20 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         }
       }
       mx = quad_row_max(mx);
+      if constexpr (FULL) mx *= rs;
       const float m_new = fmaxf(m_run[nt], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = fast_exp2(m_run[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
       m_run[nt] = m_new;
+      const float e_add = log2_pmul - m_safe;
+      const float e_mul = FULL ? rs : 1.f;
       float psum = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        float p0 = fast_exp2(s[nt][j][0] - m_safe);
-        float p1 = fast_exp2(s[nt][j][1] - m_safe);
-        float p2 = fast_exp2(s[nt][j][2] - m_safe);
-        float p3 = fast_exp2(s[nt][j][3] - m_safe);
+        float p0 = fast_exp2(__builtin_fmaf(s[nt][j][0], e_mul, e_add));
+        float p1 = fast_exp2(__builtin_fmaf(s[nt][j][1], e_mul, e_add));
+        float p2 = fast_exp2(__builtin_fmaf(s[nt][j][2], e_mul, e_add));
+        float p3 = fast_exp2(__builtin_fmaf(s[nt][j][3], e_mul, e_add));
         psum += (p0 + p1) + (p2 + p3);
         if constexpr (FP8MATH) {
           if constexpr (PER_TOKEN) {
@@ -624,10 +631,6 @@ void pa_partition_kernel(const PaDecodeArgs a) {
             p2 *= vs_cur[j][2];
             p3 *= vs_cur[j][3];
           }
-          p0 *= pmul;
-          p1 *= pmul;
-          p2 *= pmul;
-          p3 *= pmul;
           int hi = 0, lo = 0;
           hi = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, hi, false);
           hi = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, hi, true);
@@ -656,7 +659,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         pk[1] = pack_bf16x2(p2, p3);
         *reinterpret_cast<u32x2*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes + (16 * j + 4 * kg) * 2) = pk;
       }
-      l_run[nt] = l_run[nt] * alpha + psum;
+      l_run[nt] = l_run[nt] * alpha + psum * inv_pmul;
       const float alpha_acc = alpha * vfac;
 #pragma unroll
       for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha_acc;
@@ -739,7 +742,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 
   // ---- main loop -------------------------------------------------------------------------------------------
   // leading steps that need no masking: tok0 + 64 <= min_limit
-  int n_full = has_alibi ? 0 : (min_limit - part_start) / kStepTokens;
+  // the unmasked variant of the step scales the row maximum after taking it: only right for scales >= 0
+  bool rs_neg = false;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) rs_neg = rs_neg || rscale[nt] < 0.f;
+  int n_full = (has_alibi || __builtin_amdgcn_ballot_w64(rs_neg) != 0) ? 0 : (min_limit - part_start) / kStepTokens;
   n_full = n_full < 0 ? 0 : n_full;
   int sidx = 0;
   int tok0 = part_start;
