@@ -22,11 +22,19 @@ if HERE not in sys.path:
 
 METRIC = "µs/call + achieved KV HBM GB/s (% peak), FP8 KV, B=64 GQA8 ctx=4k"
 HBM_PEAK_GBPS = 8000.0
-PARTITION_KERNEL = "pa_partition_kernel"
 # HBM bytes per launch of the partition kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
-# the counter reads for a plain copy of known size (profiles/pa_partition_kernel_c2_hbm_traffic.md);
-# keyed by (workload, partition size) because the partial-output traffic depends on the partitioning
-HBM_TRAFFIC_BYTES = {("c2_fp8_b64_ctx4k", 4096): 541_300_000}
+# the counter reads for a plain copy of known size (profiles/pa_partition_kernel_c2_hbm_traffic.md,
+# profiles/pa_partition_shared_kernel_c5_hbm_traffic.md); keyed by (workload, partition size) because the
+# partial-output traffic depends on the partitioning
+HBM_TRAFFIC_BYTES = {("c2_fp8_b64_ctx4k", 4096): 541_400_000, ("c5_ragged_mix", 3840): 2_063_900_000}
+
+
+def _partition_kernel_name(wl):
+    """The kernel the library launches for this workload: more than 16 query rows per kv head over an FP8
+    cache go to the kernel whose row tiles share one pass over the pages."""
+    ge = wl.q_len * (wl.num_q_heads // wl.num_kv_heads)
+    fp8 = wl.key_cache.element_size() == 1
+    return "pa_partition_shared_kernel" if (fp8 and ge > 16) else "pa_partition_kernel"
 
 
 def _cpu_baseline(wl_cpu_sample, n_seq_sample, target_seconds=20.0):
@@ -206,7 +214,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": PARTITION_KERNEL,
+            "kernel": _partition_kernel_name(wl0),
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
