@@ -129,25 +129,29 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
                                     int32_t max_context_len, int32_t block_size, int32_t num_cus);
 
 /*
- * Stage 1: one (sequence, kv head, partition) per wave.  Gathers the partition's KV pages through
+ * Stage 1: for every (sequence, kv head, partition) gathers the partition's KV pages through
  * block_tables, computes softmax(scale * Q K^T + mask) V over the partition on MFMA and writes
  * max_logits (max of the scaled logits), exp_sums (un-normalised) and tmp_output (normalised).
  * Replaces paged_attention_decode_v2_gluon_fp8 / _large_block_fp8
  * (pa_decode_triton_gluon_fp8.py:514-1002, :27-501) and
  * _paged_attn_decode_v2_w_dot_kernel_reshape_noloop_qk (pa_decode_triton.py:26-224).
- * Partitions at or beyond ceil(context_len / partition_size) are not written.
+ * Partitions at or beyond ceil(context_len / partition_size) are not written.  When output is not NULL
+ * and there are no sinks, the output rows of every sequence with context_len <= partition_size are
+ * written here as well (their single partial is the result).
  */
 int pa_decode_partition(const PaDecodeArgs* args, void* hip_stream);
 
 /*
  * Stage 2: merges the first ceil(context_len / partition_size) partitions of every row into
- * output.  Replaces paged_attention_decode_v2_reduce_kernel
+ * output (every sequence, also those with one partition; attention sinks enter the denominator here).
+ * Replaces paged_attention_decode_v2_reduce_kernel
  * (pa_decode_triton_gluon_fp8.py:1187-1333) and _paged_attn_decode_v2_w_dot_reduce_kernel
  * (pa_decode_triton.py:227-324).
  */
 int pa_decode_reduce(const PaDecodeArgs* args, void* hip_stream);
 
-/* Both stages back to back on one stream: the body of the reference's paged_attention_decode. */
+/* Both stages back to back on one stream: the body of the reference's paged_attention_decode.  Stage 2
+ * skips the sequences stage 1 has finished, and is not launched when max_num_partitions == 1 (no sinks). */
 int pa_decode(const PaDecodeArgs* args, void* hip_stream);
 
 /*

@@ -1,5 +1,9 @@
-// Split-KV paged-attention decode for MI355X (gfx950 / CDNA4): partition kernel, reduce kernel
-// and the C ABI declared in include/pa_decode.h.
+// Split-KV paged-attention decode for MI355X (gfx950 / CDNA4): the two partition kernels, the reduce
+// kernel and the C ABI declared in include/pa_decode.h.
+//
+// pa_partition_kernel (up to 16 query rows per kv head, and every bf16 cache) is described first;
+// pa_partition_shared_kernel (17..64 rows over an FP8 cache) does the same arithmetic with the row tiles
+// of a kv head sharing one pass over the pages through LDS, and is described where it is defined.
 //
 // Work decomposition.  A workgroup of 1, 2 or 4 waves owns one item: (sequence, partition, 16-row
 // query tile, kv head).  Each wave streams a contiguous slice of the partition in steps of 64 tokens
