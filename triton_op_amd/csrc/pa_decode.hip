@@ -303,11 +303,13 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int wg_start = part * a.partition_size;
   if (wg_start >= ctx) break;
   const int wg_end = min(wg_start + a.partition_size, ctx);
-  // this wave's contiguous slice of the partition, in whole steps; a wave past the end idles until the merge
+  // The waves take the partition's 64-token steps round robin (wave w: steps w, w + WAVES, ...), so at any
+  // time the workgroup reads WAVES * 64 consecutive tokens: with large blocks that is whole 128-byte lines of
+  // every V row and long runs of every K chunk row, requested by the waves together.  A wave with no step
+  // idles until the merge.
   const int wg_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
-  const int steps_per_wave = (wg_steps + WAVES - 1) / WAVES;
-  const int part_start = wg_start + wave * steps_per_wave * kStepTokens;
-  const int part_end = min(part_start + steps_per_wave * kStepTokens, wg_end);
+  constexpr int kWaveStride = WAVES * kStepTokens;
+  const int part_start = wg_start + wave * kStepTokens;
   const bool active = part_start < wg_end;
   const int G = a.group_size;
   const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
@@ -358,7 +360,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   for (int db = 0; db < 8; ++db) v_lane_off[db] = li * v_row_bytes + 16 * db * v_row_bytes;
 
   const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
-  const int last_tile_tok = (part_end - 1) & ~15;  // first token of the last tile that holds a live token
+  const int last_tile_tok = (wg_end - 1) & ~15;  // first token of the last tile that holds a live token
 
   // page ids of the four tiles of the step that starts at token tok0 (scalar loads; tiles past the
   // last live one repeat it, so no block-table slot or page beyond the sequence is ever touched)
@@ -409,7 +411,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   };
 
   // ---- first loads go out before anything else is set up ---------------------------------------------
-  const int n_steps = (part_end - part_start + kStepTokens - 1) / kStepTokens;
+  const int n_steps = active ? (wg_steps - wave + WAVES - 1) / WAVES : 0;
   SD buf_a;  // one step of cache data, refilled in place for the next step
   if (active) {
     Pages pg0 = load_pages(part_start);
@@ -745,18 +747,19 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   };
 
   // ---- main loop -------------------------------------------------------------------------------------------
-  // leading steps that need no masking: tok0 + 64 <= min_limit
   // the unmasked variant of the step scales the row maximum after taking it: only right for scales >= 0
   bool rs_neg = false;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) rs_neg = rs_neg || rscale[nt] < 0.f;
-  int n_full = (has_alibi || __builtin_amdgcn_ballot_w64(rs_neg) != 0) ? 0 : (min_limit - part_start) / kStepTokens;
-  n_full = n_full < 0 ? 0 : n_full;
+  // leading steps of this wave that need no masking: part_start + i * stride + 64 <= min_limit
+  int n_full = 0;
+  if (!has_alibi && __builtin_amdgcn_ballot_w64(rs_neg) == 0 && min_limit - part_start >= kStepTokens)
+    n_full = (min_limit - part_start - kStepTokens) / kWaveStride + 1;
   int sidx = 0;
   int tok0 = part_start;
   if (active) {
     const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
-    Pages pg_next = load_pages(part_start + kStepTokens);
+    Pages pg_next = load_pages(part_start + kWaveStride);
     for (; sidx < n_fast; ++sidx) {
       // Waves that share a SIMD do not progress evenly by themselves (the older one wins every
       // arbitration and finishes a third earlier, leaving the SIMD half empty at the end): the further a
@@ -772,16 +775,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         else
           __builtin_amdgcn_s_setprio(0);
       }
-      const Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
+      const Pages pg_after = load_pages(tok0 + 2 * kWaveStride);
       step.template operator()<true, true>(buf_a, tok0, pg_next);
       pg_next = pg_after;
-      tok0 += kStepTokens;
+      tok0 += kWaveStride;
     }
     for (; sidx < n_steps - 1; ++sidx) {
-      const Pages pg_after = load_pages(tok0 + 2 * kStepTokens);
+      const Pages pg_after = load_pages(tok0 + 2 * kWaveStride);
       step.template operator()<false, true>(buf_a, tok0, pg_next);
       pg_next = pg_after;
-      tok0 += kStepTokens;
+      tok0 += kWaveStride;
     }
     if (n_full >= n_steps)
       step.template operator()<true, false>(buf_a, tok0, pg_next);
