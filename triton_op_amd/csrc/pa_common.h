@@ -1,0 +1,182 @@
+// Shared by the decode kernels: vector types, FP8 / bf16 conversions, scalar loads, the cross-lane
+// exchanges of the softmax, the partial-tile store and the global-to-LDS loads.  Included by exactly one
+// translation unit (pa_decode.hip), hence the unnamed namespace.
+#ifndef PA_COMMON_H_
+#define PA_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/pa_decode.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+constexpr int kHeadSize = 128;
+constexpr int kStepTokens = 64;     // tokens per pipeline step (4 tiles of 16)
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kPRowBytes = 144;     // 64 tokens * 2 B + 16 B pad per query row of the P tile
+
+union Bf16x8Bits {
+  bf16x8 v;
+  bf16x2 p[4];
+  u32x4 u;
+};
+
+// two FP8 e4m3fn bytes -> two bf16, exactly (an e4m3 value has 3 mantissa bits, bf16 keeps 7)
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t word, bool high_half) {
+  // v_cvt_pk_f32_fp8, then keep the upper 16 bits of each f32
+  f32x2 f = high_half ? __builtin_amdgcn_cvt_pk_f32_fp8((int)word, true)
+                      : __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
+  return __builtin_amdgcn_perm(__float_as_uint(f[1]), __float_as_uint(f[0]), 0x07060302u);
+}
+
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(uint32_t lo, uint32_t hi) {
+  Bf16x8Bits r;
+  r.u[0] = fp8x2_to_bf16x2(lo, false);
+  r.u[1] = fp8x2_to_bf16x2(lo, true);
+  r.u[2] = fp8x2_to_bf16x2(hi, false);
+  r.u[3] = fp8x2_to_bf16x2(hi, true);
+  return r.v;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  union {
+    bf16x2 v;
+    uint32_t u;
+  } r;
+  r.v[0] = (__bf16)a;
+  r.v[1] = (__bf16)b;
+  return r.u;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// wave-uniform 32-bit load through the scalar (constant) path: no VGPR, no vmcnt slot
+__device__ __forceinline__ int sload_i32(const int* p) {
+  return *reinterpret_cast<const __attribute__((address_space(4))) int*>(reinterpret_cast<uintptr_t>(p));
+}
+__device__ __forceinline__ float sload_f32(const float* p) {
+  return *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(p));
+}
+
+// max / sum over the four lanes {l, l^16, l^32, l^48}: v_permlane{16,32}_swap exchange 16- and
+// 32-lane halves inside the VALU (no LDS round trip)
+__device__ __forceinline__ float quad_row_max(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  u = __float_as_uint(x);
+  auto b = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_row_sum(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  u = __float_as_uint(x);
+  auto b = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// 4x4 transpose over (lane group l>>4, register): afterwards register k of lane group g holds what
+// register g of lane group k held
+__device__ __forceinline__ void quad_transpose(uint32_t (&d)[4]) {
+  auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+  auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+  auto s01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+  auto s23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+  d[0] = s01[0];
+  d[1] = s01[1];
+  d[2] = s23[0];
+  d[3] = s23[1];
+}
+
+// keep the first `n` (0..16) bytes of a 16-byte vector, zero the rest
+__device__ __forceinline__ u32x4 keep_first_bytes(u32x4 v, int n) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    int k = n - 4 * w;
+    uint32_t m = k >= 4 ? 0xffffffffu : (k <= 0 ? 0u : ((1u << (8 * k)) - 1u));
+    v[w] &= m;
+  }
+  return v;
+}
+
+// Writes one 16-row x 128-dim f32 tile of O^T (acc[db][r] = head dim 16*db + 4*kg + r of row li) as bf16
+// rows of the partial output.  The tile is transposed through a wave-private LDS buffer so that every
+// store instruction writes four whole 256-byte rows (16 bytes per lane) instead of 32-byte fragments.
+constexpr int kORowBytes = 272;  // 256 B of bf16 + 16 B pad
+__device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, char* dst,
+                                                   int64_t row_stride_bytes, char* dst2, int64_t row_stride2_bytes,
+                                                   int rows_to_write, int lane) {
+  const int li = lane & 15, kg = lane >> 4;
+#pragma unroll
+  for (int db = 0; db < 8; ++db) {
+    const f32x4 o = acc[db] * inv;
+    u32x2 pk;
+    pk[0] = pack_bf16x2(o[0], o[1]);
+    pk[1] = pack_bf16x2(o[2], o[3]);
+    *reinterpret_cast<u32x2*>(lds + li * kORowBytes + (16 * db + 4 * kg) * 2) = pk;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * i + kg;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(lds + r * kORowBytes + li * 16);
+    if (r < rows_to_write) {
+      *reinterpret_cast<u32x4*>(dst + (int64_t)r * row_stride_bytes + li * 16) = v;
+      if (dst2) *reinterpret_cast<u32x4*>(dst2 + (int64_t)r * row_stride2_bytes + li * 16) = v;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// Global memory -> LDS without passing through registers: lane i's 16 (4) bytes land at lds_offset + 16 (4) * i.
+// The loads count in vmcnt like any other vector load, but the compiler does not see them: whoever reads
+// the LDS bytes waits with dma_wait<N>() (at most N vector memory operations still outstanding) first.
+__device__ __forceinline__ void dma_load16(const void* gptr, uint32_t lds_offset) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_offset) : "memory");
+}
+__device__ __forceinline__ void dma_load4(const void* gptr, uint32_t lds_offset) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(lds_offset) : "memory");
+}
+// the same with the address split into a wave-uniform base and a 32-bit per-lane byte offset
+__device__ __forceinline__ void dma_load16(const void* base, uint32_t lane_offset, uint32_t lds_offset) {
+  // the base is wave-uniform by construction; readfirstlane makes the compiler keep it in scalar registers
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  // (the builtin returns a signed int: widen through uint32_t, or a low word with bit 31 set would smear
+  // ones over the high word)
+  const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+  const uint64_t sb = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(sb),
+               "s"(lds_offset)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
+  return (uint32_t)reinterpret_cast<uintptr_t>(
+      (const __attribute__((address_space(3))) char*)(const char*)p);
+}
+
+}  // namespace
+
+#endif  // PA_COMMON_H_

@@ -1,0 +1,777 @@
+// pa_partition_kernel: stage 1 for up to 16 query rows per kv head (and for every bf16 cache).
+//
+// Work decomposition.  A workgroup of 1, 2 or 4 waves owns one item: (sequence, partition, 16-row
+// query tile, kv head).  The waves take the partition's steps of 64 tokens (four 16-token tiles) round
+// robin, each with private online-softmax state (m, l, O), and merge through LDS at the end.  A sequence that fits in one partition gets its final output from this kernel directly.
+//
+//   K tile  (16 tokens x 128 dims): every lane loads 16 bytes = one [token][16-byte chunk] cell of
+//           the cache; lanes 0-15 are the 16 tokens of a page, lane>>4 picks the chunk row, so a
+//           wave load covers 4 x 256 contiguous bytes in storage order.  The dot product does not care
+//           in which order the head dimension is summed, so the query operand is built in the order
+//           the loads deliver it.
+//   S^T = K Q^T: tokens are the M rows, query rows (GQA group x MTP position, padded to 16) are
+//           the N columns, so a lane ends up with 4 tokens of ONE query row per tile and the softmax
+//           max/sum need only two cross-lane steps (lane^16, lane^32).
+//   V tile  (128 dims x 16 tokens): every lane loads 16 bytes = 16 tokens of one head dim, lanes
+//           0-15 are 16 consecutive dims (256 contiguous bytes with block 16), lane>>4 picks one of
+//           the four tiles of the step.  O^T = V^T P^T accumulates in 8 MFMA tiles of [16 dims x 16 rows].
+//
+// FP8 cache: the cache bytes are MFMA operands as they are (v_mfma_f32_16x16x128_f8f6f4 for Q K^T,
+// v_mfma_f32_16x16x32_fp8_fp8 for P V); the bf16 query and P are each carried as an FP8 head plus an
+// FP8 residual (x*c = hi + lo, every product exact in the f32 accumulator), about 2^-8 relative per
+// element, so there is no FP8->bf16 conversion work at all; P reaches the B-operand layout through a 4x4
+// (lane group x register) transpose with v_permlane{16,32}_swap, not through LDS.  Per-tensor scales
+// fold into the softmax scale (K) and the epilogue (V); per-token scales multiply S and P in f32.
+// bf16 cache: bf16 MFMA (v_mfma_f32_16x16x32_bf16), P through a wave-private LDS tile.
+#ifndef PA_PARTITION_KERNEL_H_
+#define PA_PARTITION_KERNEL_H_
+
+#include "pa_common.h"
+
+namespace {
+
+// One step's worth of cache data, as loaded (still FP8 / bf16 bit patterns).
+template <int KVT, bool PER_TOKEN>
+struct StepData {
+  static constexpr int NKL = KVT == PA_DTYPE_FP8_E4M3FN ? 2 : 4;  // 16-byte K loads per lane per tile
+  static constexpr int NVL = KVT == PA_DTYPE_FP8_E4M3FN ? 1 : 2;  // 16-byte V loads per lane per 16 dims
+  u32x4 k[4][NKL];
+  u32x4 v[8][NVL];
+  f32x4 ks[PER_TOKEN ? 4 : 1];
+  f32x4 vs[PER_TOKEN ? 4 : 1];
+};
+
+// The partition kernel.  OCC is the number of waves per SIMD the register budget is cut for.
+//
+// Software pipeline of one wave (each line is issued in order; loads return in order):
+//   QK(s)      needs K(s)            -> then K(s+1) is loaded into the registers K(s) just left
+//   softmax(s)                          (K(s+1) and V(s) in flight)
+//   PV(s)      needs V(s)            -> then V(s+1) is loaded into the registers V(s) just left
+// so about one step (16 KiB) of cache data per wave is in flight at any time without a second
+// register copy.  Steps that need no masking and have a successor run in a branch-free loop, so
+// the compiler's vmcnt waits stay partial; the last step(s) go through the masked variants.
+//
+// BS16 (block size 16) turns every stride inside a page into a compile-time constant, so the loads
+// of a tile share one address register pair and differ by immediate offsets.
+constexpr int kQueueMaxSeqs = 2048;  // sequences the item table of the queued launch can hold
+
+template <int NT, int KVT, bool PER_TOKEN, bool BS16, int WAVES, int OCC, bool QUEUE>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void pa_partition_kernel(const PaDecodeArgs a) {
+  constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
+  constexpr bool FP8MATH = kFp8;  // an FP8 cache is multiplied on the FP8 MFMAs, a bf16 cache on the bf16 ones
+  constexpr int esz = kFp8 ? 1 : 2;
+  typedef StepData<KVT, PER_TOKEN> SD;
+
+  __shared__ __attribute__((aligned(16))) char p_lds[FP8MATH ? 1 : WAVES][FP8MATH ? 1 : NT][FP8MATH ? 16 : 16 * kPRowBytes];
+  __shared__ __attribute__((aligned(16))) char o_lds[1][16 * kORowBytes];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15;
+  const int kg = lane >> 4;
+
+  // ---- which (sequence, head, partition): all wave-uniform -----------------------------------------
+  const int P = a.max_num_partitions;
+  const int Hkv = a.num_kv_heads;
+  // The WAVES waves of a workgroup share one item: (sequence, partition, group of NT 16-row query tiles,
+  // kv head).  The head varies fastest, so the workgroups that stream the same pages (the other heads, and
+  // the other row tiles of the same head, 8 ids apart with 8 kv heads: the same XCD and L2) run together.
+  const int Ge = a.q_len * a.group_size;  // rows per kv head in the buffers
+  const int RT = (Ge + 16 * NT - 1) / (16 * NT);
+
+  // QUEUE: a resident grid of workgroups pulls live items from a counter in the caller's workspace.  Only
+  // partitions a sequence reaches and row tiles that hold real query rows are items, so a ragged batch
+  // launches no workgroup that would exit at once (each of those still costs a wave slot for a
+  // microsecond).  Every workgroup builds, once, the exclusive prefix sum of the per-sequence item counts
+  // in LDS and decodes an item index by binary search in it.
+  __shared__ int q_cum[QUEUE ? kQueueMaxSeqs + 1 : 1];
+  __shared__ int q_ctx[QUEUE ? kQueueMaxSeqs : 1];
+  __shared__ int q_tiles[QUEUE ? kQueueMaxSeqs : 1];
+  __shared__ int q_item;
+  int total_items = 0;
+  if constexpr (QUEUE) {
+    if (wave == 0) {
+      int running = 0;
+      for (int b0 = 0; b0 < a.num_seqs; b0 += 64) {
+        const int bb = b0 + lane;
+        const int c = bb < a.num_seqs ? a.context_lens[bb] : 0;
+        int np = (c + a.partition_size - 1) / a.partition_size;
+        np = np < 0 ? 0 : (np > P ? P : np);
+        const int ql = bb < a.num_seqs ? (a.q_lens ? a.q_lens[bb] : a.q_len) : 0;
+        int tiles = (ql * a.group_size + 16 * NT - 1) / (16 * NT);
+        tiles = tiles > RT ? RT : tiles;
+        const int n = np * tiles;
+        int x = n;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int y = __shfl_up(x, d);
+          if (lane >= d) x += y;
+        }
+        if (bb < a.num_seqs) {
+          q_cum[bb] = running + x - n;
+          q_ctx[bb] = c;
+          q_tiles[bb] = tiles;
+        }
+        running += __builtin_amdgcn_readlane(x, 63);
+      }
+      if (lane == 0) q_cum[a.num_seqs] = running;
+    }
+    __syncthreads();
+    total_items = q_cum[a.num_seqs] * Hkv;
+  }
+
+  for (;;) {  // one pass without the queue
+  int h, rt, b, part, tiles_b = RT;
+  if constexpr (QUEUE) {
+    if (threadIdx.x == 0) q_item = atomicAdd(a.workspace, 1);
+    __syncthreads();
+    const int item = __builtin_amdgcn_readfirstlane(q_item);
+    __syncthreads();  // everybody has read q_item (and is done with the LDS buffers of the previous item)
+    if (item >= total_items) break;
+    h = item % Hkv;
+    const int j = item / Hkv;
+    int lo = 0, hi = a.num_seqs;  // q_cum[lo] <= j < q_cum[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (__builtin_amdgcn_readfirstlane(q_cum[mid]) <= j)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    b = lo;
+    tiles_b = __builtin_amdgcn_readfirstlane(q_tiles[b]);
+    const int local = j - __builtin_amdgcn_readfirstlane(q_cum[b]);
+    part = local / tiles_b;
+    rt = local - part * tiles_b;
+  } else {
+    // The partition index varies slowest: in a ragged batch the partitions that only the longest
+    // sequences reach (workgroups that exit at once for everybody else) come last.
+    const long long wid = blockIdx.x;
+    h = (int)(wid % Hkv);
+    rt = (int)((wid / Hkv) % RT);
+    b = (int)((wid / ((long long)Hkv * RT)) % a.num_seqs);
+    part = (int)(wid / ((long long)Hkv * RT * a.num_seqs));
+  }
+  const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
+  do {  // the body of one item; `break` leaves it
+
+  const int ctx = sload_i32(a.context_lens + b);
+  const int wg_start = part * a.partition_size;
+  if (wg_start >= ctx) break;
+  const int wg_end = min(wg_start + a.partition_size, ctx);
+  // The waves take the partition's 64-token steps round robin (wave w: steps w, w + WAVES, ...), so at any
+  // time the workgroup reads WAVES * 64 consecutive tokens: with large blocks that is whole 128-byte lines of
+  // every V row and long runs of every K chunk row, requested by the waves together.  A wave with no step
+  // idles until the merge.
+  const int wg_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
+  constexpr int kWaveStride = WAVES * kStepTokens;
+  const int part_start = wg_start + wave * kStepTokens;
+  const bool active = part_start < wg_end;
+  const int G = a.group_size;
+  const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
+  const int rows_valid = qb * G;
+  if (row0 >= rows_valid) {
+    // only padding rows (a ragged batch): nothing to stream; the rows read as "no visible key"
+    if (wave == 0) {
+      const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+      char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                        (int64_t)part * a.stride_tmp_p) * 2;
+      char* op = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+      const bool dir = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
+      for (int r = row0 + kg; r < row0 + 16 * NT && r < Ge; r += 4) {
+        if (li == 0) {
+          a.max_logits[eo + r] = -INFINITY;
+          a.exp_sums[eo + r] = 0.f;
+        }
+        *reinterpret_cast<u32x4*>(tp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
+        if (dir) *reinterpret_cast<u32x4*>(op + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
+      }
+    }
+    break;
+  }
+
+  // ---- cache addressing -------------------------------------------------------------------------------
+  const int log2_bs = 31 - __builtin_clz(a.block_size);
+  const int bs_mask = a.block_size - 1;
+  const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h * esz;
+  const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h * esz;
+  const int64_t k_block_bytes = a.stride_k_b * esz;
+  const int64_t v_block_bytes = a.stride_v_b * esz;
+  const float* ksbase = PER_TOKEN ? a.key_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  const float* vsbase = PER_TOKEN ? a.value_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  const uint32_t k_chunk_bytes = BS16 ? 256u : (uint32_t)(a.stride_k_c * esz);
+  uint32_t k_lane_off[SD::NKL];  // per-lane byte offset of K load ld inside a tile
+#pragma unroll
+  for (int ld = 0; ld < SD::NKL; ++ld) k_lane_off[ld] = (uint32_t)(kg * k_chunk_bytes + li * 16) + 4 * ld * k_chunk_bytes;
+  // V: byte offset of this lane's head dim inside a tile, distance of the second 8-token half
+  // (bf16 only) and, for the transposed layout, of consecutive 16-token tiles of a page
+  // (with block size 16 the plain and the transposed FP8 layouts are the same bytes; for bf16 they
+  // differ, so the constant-stride form is used for the plain layout only)
+  const bool vt = a.v_transposed;
+  const uint32_t v_row_bytes = BS16 ? 16u * esz : (vt ? 16u : (uint32_t)(a.stride_v_2 * esz));
+  const uint32_t v_half_bytes = BS16 ? 16u : (vt ? (uint32_t)(a.stride_v_2 * esz) : 16u);
+  const int64_t v_tile_bytes = BS16 ? 16 * esz : (vt ? a.stride_v_2 * esz * esz : 16 * esz);
+  uint32_t v_lane_off[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) v_lane_off[db] = li * v_row_bytes + 16 * db * v_row_bytes;
+
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const int last_tile_tok = (wg_end - 1) & ~15;  // first token of the last tile that holds a live token
+
+  // page ids of the four tiles of the step that starts at token tok0 (scalar loads; tiles past the
+  // last live one repeat it, so no block-table slot or page beyond the sequence is ever touched)
+  struct Pages {
+    int p[4];
+    int off[4];  // token offset of the tile inside its page
+  };
+  auto load_pages = [&](int tok0) {
+    Pages pg;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int t = tok0 + 16 * j;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      pg.p[j] = sload_i32(bt + (t >> log2_bs));
+      pg.off[j] = t & bs_mask;
+    }
+    return pg;
+  };
+  auto issue_k = [&](SD& sd, const Pages& pg) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const char* tb = kbase + (int64_t)pg.p[j] * k_block_bytes + (int64_t)pg.off[j] * 16;
+#pragma unroll
+      for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16(tb + k_lane_off[ld]);
+      if constexpr (PER_TOKEN) {
+        const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + pg.off[j] + 4 * kg;
+        sd.ks[j] = *reinterpret_cast<const f32x4*>(ksbase + so);
+      }
+    }
+  };
+  auto issue_v = [&](SD& sd, const Pages& pg) {
+    // lane group kg owns tile kg of the step
+    const int page = kg == 0 ? pg.p[0] : (kg == 1 ? pg.p[1] : (kg == 2 ? pg.p[2] : pg.p[3]));
+    const int off = kg == 0 ? pg.off[0] : (kg == 1 ? pg.off[1] : (kg == 2 ? pg.off[2] : pg.off[3]));
+    const char* tb = vbase + (int64_t)page * v_block_bytes + (int64_t)(off >> 4) * v_tile_bytes;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < SD::NVL; ++hf) sd.v[db][hf] = load16(tb + v_lane_off[db] + hf * v_half_bytes);
+    }
+    if constexpr (PER_TOKEN) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + pg.off[j] + 4 * kg;
+        sd.vs[j] = *reinterpret_cast<const f32x4*>(vsbase + so);
+      }
+    }
+  };
+
+  // ---- first loads go out before anything else is set up ---------------------------------------------
+  const int n_steps = active ? (wg_steps - wave + WAVES - 1) / WAVES : 0;
+  SD buf_a;  // one step of cache data, refilled in place for the next step
+  if (active) {
+    Pages pg0 = load_pages(part_start);
+    issue_k(buf_a, pg0);
+    issue_v(buf_a, pg0);
+  }
+
+  // ---- per-lane row bookkeeping -------------------------------------------------------------------------
+  int limit[NT];      // number of visible keys of this lane's query row
+  float slope2[NT];   // ALiBi slope * log2e
+  const bool has_alibi = a.alibi_slopes != nullptr;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int row = row0 + 16 * nt + li;
+    int t = row / G;
+    limit[nt] = row < rows_valid ? ctx - (qb - 1 - t) : 0;
+    slope2[nt] = 0.f;
+    if (has_alibi && row < rows_valid) slope2[nt] = a.alibi_slopes[h * G + (row - t * G)] * kLog2e;
+  }
+  const int min_limit = ctx - (qb - 1);  // keys below this index are visible to every real row
+
+  // ---- query: B operand of S^T = K Q^T --------------------------------------------------------------------
+  // k-step s of a tile covers, for lane group kg, the 8 head dims the K load puts in that slot.
+  // Rows past the last real one are loaded from row 0 and zeroed, which keeps this branch-free.
+  bf16x8 qreg[NT][4];
+  {
+    const char* q_ptr = (const char*)a.query;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int row = row0 + 16 * nt + li;
+      const bool ok = row < rows_valid;
+      const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (ok ? row : 0)) * a.stride_q_h;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
+        Bf16x8Bits q;
+        if (a.query_dtype == PA_DTYPE_BF16) {
+          q.u = load16(q_ptr + (e0 + dim) * 2);
+        } else {
+          u32x2 raw = *reinterpret_cast<const u32x2*>(q_ptr + e0 + dim);
+          q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
+        }
+        if (!ok) q.u = u32x4{0, 0, 0, 0};
+        qreg[nt][s] = q.v;
+      }
+    }
+  }
+  // per-row query scale (FP8 query) multiplies the logits of that row
+  float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
+  if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
+    k_tensor_scale = sload_f32(a.key_scale);
+    v_tensor_scale = sload_f32(a.value_scale);
+  }
+  const float scale2 = a.softmax_scale * k_tensor_scale * kLog2e;
+  float rscale[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int row = row0 + 16 * nt + li;
+    float qs = 1.f;
+    if (a.query_quant_mode == PA_QUANT_PER_TENSOR) qs = sload_f32(a.query_scale);
+    if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row < rows_valid)
+      qs = a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
+    rscale[nt] = scale2 * qs;
+  }
+  // FP8 math: q * cq = hi + lo with hi, lo in e4m3 (|q * cq| <= 224); the logits are divided by cq again
+  i32x8 qhi[FP8MATH ? NT : 1], qlo[FP8MATH ? NT : 1];
+  if constexpr (FP8MATH) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      float f[32];
+      float amax = 0.f;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        Bf16x8Bits q;
+        q.v = qreg[nt][s4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          f[8 * s4 + 2 * e] = bf16_bits_to_f32(q.u[e] & 0xffffu);
+          f[8 * s4 + 2 * e + 1] = __uint_as_float(q.u[e] & 0xffff0000u);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(f[e]));
+      amax = quad_row_max(amax);
+      const float cq = amax > 0.f ? 224.f / amax : 1.f;
+      rscale[nt] *= amax > 0.f ? amax * (1.f / 224.f) : 1.f;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        const float x0 = f[4 * w] * cq, x1 = f[4 * w + 1] * cq, x2 = f[4 * w + 2] * cq, x3 = f[4 * w + 3] * cq;
+        int hi = 0, lo = 0;
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, hi, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(x2, x3, hi, true);
+        const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+        const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(x0 - b01[0], x1 - b01[1], lo, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(x2 - b23[0], x3 - b23[1], lo, true);
+        qhi[nt][w] = hi;
+        qlo[nt][w] = lo;
+      }
+    }
+  }
+  float v_run = 1e-30f;  // FP8 math with per-token V scales: running max of the scales seen so far
+
+  float m_run[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
+  float l_run[NT];      // this lane's share of the running sum of exp2(s - m)
+  f32x4 acc[NT][8];     // O^T: acc[nt][db][r] is head dim 16*db + 4*kg + r of query row 16*nt + li
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    m_run[nt] = -INFINITY;
+    l_run[nt] = 0.f;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  char* plds = &p_lds[wave][0][0];
+
+  // ---- one step of 64 tokens ------------------------------------------------------------------------------
+  // FULL: every token of the step is visible to every row and there is no ALiBi term.
+  // PREFETCH: a next step exists; its K and V are requested as soon as this step's are consumed.
+  auto step = [&]<bool FULL, bool PREFETCH>(SD& sd, int tok0, const Pages& pg_next) {
+    // S^T tiles
+    f32x4 s[NT][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) s[nt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (FP8MATH) {
+        const i32x8 ka = {(int)sd.k[j][0][0], (int)sd.k[j][0][1], (int)sd.k[j][0][2], (int)sd.k[j][0][3],
+                          (int)sd.k[j][1][0], (int)sd.k[j][1][1], (int)sd.k[j][1][2], (int)sd.k[j][1][3]};
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          s[nt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi[nt], s[nt][j], 0, 0, 0, 0, 0, 0);
+          s[nt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo[nt], s[nt][j], 0, 0, 0, 0, 0, 0);
+        }
+      } else
+#pragma unroll
+      for (int ld = 0; ld < SD::NKL; ++ld) {
+        Bf16x8Bits ka;
+        ka.u = sd.k[j][ld];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          s[nt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka.v, qreg[nt][ld], s[nt][j], 0, 0, 0);
+      }
+    }
+    f32x4 ks_cur[PER_TOKEN ? 4 : 1];
+    if constexpr (PER_TOKEN) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ks_cur[j] = sd.ks[j];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREFETCH) issue_k(sd, pg_next);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // FP8 math, per-token V scales: P carries v_scale / v_run (<= 1); the accumulator is kept in units
+    // of the running maximum v_run
+    // FP8 math: P is produced already multiplied by pmul = 256 / v_run; log2(pmul) rides in the exponent's
+    // additive term, so the factor costs nothing per element
+    float vfac = 1.f, log2_pmul = FP8MATH ? 8.f : 0.f, inv_pmul = FP8MATH ? 1.f / 256.f : 1.f;
+    f32x4 vs_cur[(PER_TOKEN && FP8MATH) ? 4 : 1];
+    if constexpr (PER_TOKEN && FP8MATH) {
+      float vmx = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vs_cur[j] = sd.vs[j];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (!FULL) {
+            const int col = tok0 + 16 * j + 4 * kg + r;
+            vs_cur[j][r] = col < ctx ? vs_cur[j][r] : 0.f;
+          }
+          vmx = fmaxf(vmx, vs_cur[j][r]);
+        }
+      }
+      vmx = quad_row_max(vmx);
+      const float v_new = fmaxf(v_run, vmx);
+      vfac = v_new == v_run ? 1.f : v_run * __builtin_amdgcn_rcpf(v_new);
+      log2_pmul = 8.f - __builtin_amdgcn_logf(v_new);
+      inv_pmul = v_new * (1.f / 256.f);
+      v_run = v_new;
+    }
+    uint32_t ph[FP8MATH ? NT : 1][4], pl[FP8MATH ? NT : 1][4];  // FP8 math: P head / residual, 4 tokens per dword
+
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float rs = rscale[nt];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          // FULL: the row's scale (>= 0 on this path) is applied inside the exponent's fma, and to the maximum once
+          float v = s[nt][j][r];
+          if constexpr (PER_TOKEN) v *= ks_cur[j][r];
+          if constexpr (!FULL) {
+            const int col = tok0 + 16 * j + 4 * kg + r;
+            v = v * rs + slope2[nt] * (float)(col - ctx + 1);
+            v = col < limit[nt] ? v : -INFINITY;
+          }
+          s[nt][j][r] = v;
+          mx = fmaxf(mx, v);
+        }
+      }
+      mx = quad_row_max(mx);
+      if constexpr (FULL) mx *= rs;
+      const float m_new = fmaxf(m_run[nt], mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
+      m_run[nt] = m_new;
+      const float e_add = log2_pmul - m_safe;
+      const float e_mul = FULL ? rs : 1.f;
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float p0 = fast_exp2(__builtin_fmaf(s[nt][j][0], e_mul, e_add));
+        float p1 = fast_exp2(__builtin_fmaf(s[nt][j][1], e_mul, e_add));
+        float p2 = fast_exp2(__builtin_fmaf(s[nt][j][2], e_mul, e_add));
+        float p3 = fast_exp2(__builtin_fmaf(s[nt][j][3], e_mul, e_add));
+        psum += (p0 + p1) + (p2 + p3);
+        if constexpr (FP8MATH) {
+          if constexpr (PER_TOKEN) {
+            p0 *= vs_cur[j][0];
+            p1 *= vs_cur[j][1];
+            p2 *= vs_cur[j][2];
+            p3 *= vs_cur[j][3];
+          }
+          int hi = 0, lo = 0;
+          hi = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, hi, false);
+          hi = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, hi, true);
+          const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+          const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+          lo = __builtin_amdgcn_cvt_pk_fp8_f32(p0 - b01[0], p1 - b01[1], lo, false);
+          lo = __builtin_amdgcn_cvt_pk_fp8_f32(p2 - b23[0], p3 - b23[1], lo, true);
+          ph[nt][j] = (uint32_t)hi;
+          pl[nt][j] = (uint32_t)lo;
+          continue;
+        }
+        if constexpr (PER_TOKEN) {
+          // a masked token's scale may be stale memory (NaN): its weight must stay exactly 0
+          f32x4 vsc = sd.vs[j];
+          if constexpr (!FULL) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vsc[r] = s[nt][j][r] == -INFINITY ? 0.f : vsc[r];
+          }
+          p0 *= vsc[0];
+          p1 *= vsc[1];
+          p2 *= vsc[2];
+          p3 *= vsc[3];
+        }
+        u32x2 pk;
+        pk[0] = pack_bf16x2(p0, p1);
+        pk[1] = pack_bf16x2(p2, p3);
+        *reinterpret_cast<u32x2*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes + (16 * j + 4 * kg) * 2) = pk;
+      }
+      l_run[nt] = l_run[nt] * alpha + psum * inv_pmul;
+      const float alpha_acc = alpha * vfac;
+#pragma unroll
+      for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha_acc;
+    }
+
+    if constexpr (!FULL) {
+      // zero the V bytes of tokens at or beyond ctx (stale cache contents may decode to NaN)
+      int nvalid = ctx - (tok0 + 16 * kg);
+      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        if constexpr (kFp8) {
+          sd.v[db][0] = keep_first_bytes(sd.v[db][0], nvalid);
+        } else {
+          sd.v[db][0] = keep_first_bytes(sd.v[db][0], 2 * (nvalid > 8 ? 8 : nvalid));
+          sd.v[db][1] = keep_first_bytes(sd.v[db][1], 2 * (nvalid > 8 ? nvalid - 8 : 0));
+        }
+      }
+    }
+
+    if constexpr (FP8MATH) {
+      // lane group kg holds, per tile j, tokens 4kg..4kg+3; the B operand of O^T += V^T P^T wants lane
+      // group kg to hold all 16 tokens of tile kg: a 4x4 transpose over (lane group, register)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        quad_transpose(ph[nt]);
+        quad_transpose(pl[nt]);
+      }
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int db = 0; db < 8; ++db) {
+          const long va = (long)(((uint64_t)sd.v[db][0][2 * hf + 1] << 32) | sd.v[db][0][2 * hf]);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const long bh = (long)(((uint64_t)ph[nt][2 * hf + 1] << 32) | ph[nt][2 * hf]);
+            const long bl = (long)(((uint64_t)pl[nt][2 * hf + 1] << 32) | pl[nt][2 * hf]);
+            acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(va, bh, acc[nt][db], 0, 0, 0);
+            acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(va, bl, acc[nt][db], 0, 0, 0);
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PREFETCH) issue_v(sd, pg_next);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
+
+    // the P tile is written and read by this wave only; LDS operations of one wave complete in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // O^T += V^T P^T
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      bf16x8 pb[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        Bf16x8Bits t;
+        t.u = *reinterpret_cast<const u32x4*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes +
+                                              (16 * kg + 8 * hf) * 2);
+        pb[nt] = t.v;
+      }
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        Bf16x8Bits va;
+        va.u = sd.v[db][hf];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[nt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb[nt], acc[nt][db], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREFETCH) issue_v(sd, pg_next);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---- main loop -------------------------------------------------------------------------------------------
+  // the unmasked variant of the step scales the row maximum after taking it: only right for scales >= 0
+  bool rs_neg = false;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) rs_neg = rs_neg || rscale[nt] < 0.f;
+  // leading steps of this wave that need no masking: part_start + i * stride + 64 <= min_limit
+  int n_full = 0;
+  if (!has_alibi && __builtin_amdgcn_ballot_w64(rs_neg) == 0 && min_limit - part_start >= kStepTokens)
+    n_full = (min_limit - part_start - kStepTokens) / kWaveStride + 1;
+  int sidx = 0;
+  int tok0 = part_start;
+  if (active) {
+    const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
+    Pages pg_next = load_pages(part_start + kWaveStride);
+    for (; sidx < n_fast; ++sidx) {
+      // Waves that share a SIMD do not progress evenly by themselves (the older one wins every
+      // arbitration and finishes a third earlier, leaving the SIMD half empty at the end): the further a
+      // wave is from its end, the higher its issue priority.
+      {
+        const int rem4 = (n_steps - sidx) * 4 / n_steps;
+        if (rem4 >= 3)
+          __builtin_amdgcn_s_setprio(3);
+        else if (rem4 == 2)
+          __builtin_amdgcn_s_setprio(2);
+        else if (rem4 == 1)
+          __builtin_amdgcn_s_setprio(1);
+        else
+          __builtin_amdgcn_s_setprio(0);
+      }
+      const Pages pg_after = load_pages(tok0 + 2 * kWaveStride);
+      step.template operator()<true, true>(buf_a, tok0, pg_next);
+      pg_next = pg_after;
+      tok0 += kWaveStride;
+    }
+    for (; sidx < n_steps - 1; ++sidx) {
+      const Pages pg_after = load_pages(tok0 + 2 * kWaveStride);
+      step.template operator()<false, true>(buf_a, tok0, pg_next);
+      pg_next = pg_after;
+      tok0 += kWaveStride;
+    }
+    if (n_full >= n_steps)
+      step.template operator()<true, false>(buf_a, tok0, pg_next);
+    else
+      step.template operator()<false, false>(buf_a, tok0, pg_next);
+  }
+
+  // ---- epilogue ------------------------------------------------------------------------------------------------
+  // max_logits holds the maximum of the scaled logits in the natural-log domain, exp_sums the
+  // un-normalised sum, tmp_output the normalised bf16 partial.  For a sequence that fits in one partition the
+  // partial is the result, and it is written to output as well.
+  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+  char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                     (int64_t)part * a.stride_tmp_p) * 2;
+  // a sequence that fits in one partition needs no merge: its partial is the result
+  const bool direct = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
+  char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+  const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
+  float l_tot[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    l_tot[nt] = quad_row_sum(l_run[nt]);
+    if (row0 + 16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
+      l_tot[nt] = 0.f;
+      m_run[nt] = -INFINITY;
+    }
+  }
+  if constexpr (WAVES == 1) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int row = row0 + 16 * nt + li;
+      const float inv = l_tot[nt] > 0.f ? v_tensor_scale * acc_unit / l_tot[nt] : 0.f;
+      if (row < Ge && kg == 0) {
+        a.max_logits[es_off + row] = m_run[nt] * (1.0f / kLog2e);
+        a.exp_sums[es_off + row] = l_tot[nt];
+      }
+      store_partial_tile(&o_lds[0][0], acc[nt], inv, tmp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2,
+                         a.stride_tmp_g * 2, direct ? outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2 : nullptr,
+                         a.stride_out_h * 2, Ge - row0 - 16 * nt, lane);
+    }
+  } else {
+    // merge the waves' (m, l, O): every wave holds the same (row, head dim) in the same lane and register,
+    // so the merge is lane-wise; wave w merges head-dim blocks [w*8/WAVES, (w+1)*8/WAVES)
+    __shared__ float mg_m[WAVES][NT * 16];
+    __shared__ float mg_l[WAVES][NT * 16];
+    __shared__ f32x4 mg_acc[WAVES][NT][8][64];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (kg == 0) {
+        mg_m[wave][16 * nt + li] = m_run[nt];
+        mg_l[wave][16 * nt + li] = l_tot[nt];
+      }
+#pragma unroll
+      for (int db = 0; db < 8; ++db) mg_acc[wave][nt][db][lane] = acc[nt][db] * acc_unit;
+    }
+    __syncthreads();
+    constexpr int DBW = 8 / WAVES;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int lrow = 16 * nt + li;
+      const int row = row0 + lrow;
+      float M = -INFINITY;
+#pragma unroll
+      for (int w2 = 0; w2 < WAVES; ++w2) M = fmaxf(M, mg_m[w2][lrow]);
+      const float M_safe = M == -INFINITY ? 0.f : M;
+      float e[WAVES];
+      float L = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < WAVES; ++w2) {
+        e[w2] = fast_exp2(mg_m[w2][lrow] - M_safe);
+        L += mg_l[w2][lrow] * e[w2];
+      }
+      const float inv = L > 0.f ? v_tensor_scale / L : 0.f;
+#pragma unroll
+      for (int d = 0; d < DBW; ++d) {
+        const int db = wave * DBW + d;
+        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w2 = 0; w2 < WAVES; ++w2) o += mg_acc[w2][nt][db][lane] * e[w2];
+        o *= inv;
+        u32x2 pk;
+        pk[0] = pack_bf16x2(o[0], o[1]);
+        pk[1] = pack_bf16x2(o[2], o[3]);
+        *reinterpret_cast<u32x2*>(&o_lds[0][0] + li * kORowBytes + (16 * db + 4 * kg) * 2) = pk;
+      }
+      if (wave == 0 && kg == 0 && row < Ge) {
+        a.max_logits[es_off + row] = M * (1.0f / kLog2e);
+        a.exp_sums[es_off + row] = L;
+      }
+      __syncthreads();
+      for (int i = wave; i < 4; i += WAVES) {
+        const int r = 4 * i + kg;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(&o_lds[0][0] + r * kORowBytes + li * 16);
+        if (r < Ge - row0 - 16 * nt) {
+          *reinterpret_cast<u32x4*>(tmp + (int64_t)(row0 + 16 * nt + r) * a.stride_tmp_g * 2 + li * 16) = v;
+          if (direct)
+            *reinterpret_cast<u32x4*>(outp + (int64_t)(row0 + 16 * nt + r) * a.stride_out_h * 2 + li * 16) = v;
+        }
+      }
+      if (nt + 1 < NT) __syncthreads();
+    }
+  }
+  if constexpr (QUEUE) {
+    // rows of padding query positions beyond the last real tile: this workgroup fills them
+    if (rt == tiles_b - 1 && wave == 0) {
+      for (int r = 16 * NT * tiles_b + kg; r < Ge; r += 4) {
+        if (li == 0) {
+          a.max_logits[es_off + r] = -INFINITY;
+          a.exp_sums[es_off + r] = 0.f;
+        }
+        *reinterpret_cast<u32x4*>(tmp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
+        if (direct) *reinterpret_cast<u32x4*>(outp + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
+      }
+    }
+  }
+  } while (0);
+  if constexpr (!QUEUE) break;
+  }  // for (;;)
+  if constexpr (QUEUE) {
+    // the last workgroup out leaves the workspace as it found it: zero
+    if (threadIdx.x == 0) {
+      __threadfence();
+      if (atomicAdd(a.workspace + 1, 1) == (int)gridDim.x - 1) {
+        a.workspace[0] = 0;
+        a.workspace[1] = 0;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+#endif  // PA_PARTITION_KERNEL_H_

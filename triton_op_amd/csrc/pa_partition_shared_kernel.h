@@ -1,0 +1,415 @@
+// pa_partition_shared_kernel: stage 1 for 17..64 query rows per kv head over an FP8 cache.
+#ifndef PA_PARTITION_SHARED_KERNEL_H_
+#define PA_PARTITION_SHARED_KERNEL_H_
+
+#include "pa_common.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// Partition kernel for more than 16 query rows per kv head (large GQA groups, MTP) over an FP8 cache.
+// The up to four 16-row query tiles of one (sequence, kv head, partition) are the four waves of ONE
+// workgroup and share a single pass over the pages.  Of every 64-token step each wave fetches a quarter
+// (K tile `wave`, V head-dim blocks 2*wave and 2*wave+1) into registers and parks it in LDS in exactly the
+// per-lane operand order of the MFMAs; after a workgroup barrier every wave reads the whole step back
+// with lane-contiguous 16-byte LDS reads.  Two LDS buffers: step s+1 travels from HBM while step s is multiplied,
+// one barrier per step.  Against one workgroup per row tile this reads every page once instead of once per
+// tile (the repeats hit the L2, but each costs a full trip through the vector memory path).
+// ---------------------------------------------------------------------------------------------
+struct StepLds {
+  u32x4 k[4][2][64];  // [tile][load][lane]: the K operand of a tile as its two loads deliver it
+  u32x4 v[4][128];    // [tile][head dim]: 16 tokens of one head dim
+  float sc[4][2][16]; // [tile][K scales, V scales][token]
+};
+
+template <bool PER_TOKEN, bool BS16, int NB, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void pa_partition_shared_kernel(const PaDecodeArgs a) {
+  __shared__ __attribute__((aligned(16))) StepLds stage[NB];  // ring of steps: NB-1 in flight, one being read
+  static_assert(sizeof(StepLds) * NB >= 4 * 16 * kORowBytes, "the output tiles reuse the stage buffers");
+  constexpr int kLoadsPerStep = PER_TOKEN ? 5 : 4;  // vector memory operations one wave issues per step
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15;
+  const int kg = lane >> 4;
+
+  // ---- which (sequence, head, partition): workgroup-uniform; head fastest, partition slowest ----------
+  const int Hkv = a.num_kv_heads;
+  const int G = a.group_size;
+  const int Ge = a.q_len * G;
+  const long long wid = blockIdx.x;
+  const int h = (int)(wid % Hkv);
+  const int b = (int)((wid / Hkv) % a.num_seqs);
+  const int part = (int)(wid / ((long long)Hkv * a.num_seqs));
+
+  const int ctx = sload_i32(a.context_lens + b);
+  const int wg_start = part * a.partition_size;
+  if (wg_start >= ctx) return;
+  const int wg_end = min(wg_start + a.partition_size, ctx);
+  const int n_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
+  const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
+  const int rows_valid = qb * G;
+  const int row0 = 16 * wave;               // this wave's query tile
+  const bool has_rows = row0 < rows_valid;  // else the wave only helps to fetch
+
+  // ---- cache addressing ----------------------------------------------------------------------------------
+  const int log2_bs = 31 - __builtin_clz(a.block_size);
+  const int bs_mask = a.block_size - 1;
+  const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h;
+  const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h;
+  const int64_t k_block_bytes = a.stride_k_b;
+  const int64_t v_block_bytes = a.stride_v_b;
+  const float* ksbase = PER_TOKEN ? a.key_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  const float* vsbase = PER_TOKEN ? a.value_scale + (int64_t)h * a.stride_kvscale_h : nullptr;
+  const uint32_t k_chunk_bytes = BS16 ? 256u : (uint32_t)a.stride_k_c;
+  uint32_t k_lane_off[2];
+#pragma unroll
+  for (int ld = 0; ld < 2; ++ld) k_lane_off[ld] = (uint32_t)(kg * k_chunk_bytes + li * 16) + 4 * ld * k_chunk_bytes;
+  const bool vt = a.v_transposed;
+  const uint32_t v_row_bytes = BS16 ? 16u : (vt ? 16u : (uint32_t)a.stride_v_2);
+  const int64_t v_tile_bytes = BS16 ? 16 : (vt ? a.stride_v_2 : 16);
+  uint32_t v_lane_off[2];  // V loads: lane = head dim (0..63, 64..127) of one tile
+#pragma unroll
+  for (int i = 0; i < 2; ++i) v_lane_off[i] = (uint32_t)(lane + 64 * i) * v_row_bytes;
+  const float* sc_lane = PER_TOKEN ? ((lane & 16) ? vsbase : ksbase) + li : nullptr;
+
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const int last_tile_tok = (wg_end - 1) & ~15;
+  // wave w fetches tile w of every step: its page id (a scalar load) and the tile's token offset inside the
+  // page.  Tiles past the last live one repeat it, so no block-table slot or page beyond the sequence is touched.
+  struct TilePage {
+    int page;
+    int off;
+  };
+  auto load_page = [&](int tok0) {
+    int t = tok0 + 16 * wave;
+    t = t > last_tile_tok ? last_tile_tok : t;
+    TilePage tp;
+    tp.page = sload_i32(bt + (t >> log2_bs));
+    tp.off = t & bs_mask;
+    return tp;
+  };
+  // this wave's quarter of the step whose page ids are pg, sent to ring slot `slot`
+  const uint32_t stage_base = lds_offset_of(&stage[0]);
+  auto fetch = [&](int slot, const TilePage& tp) {
+    const uint32_t st = stage_base + (uint32_t)slot * (uint32_t)sizeof(StepLds);
+    // every address is a wave-uniform base plus a per-lane constant
+    const int page = tp.page;
+    const int off = tp.off;
+    const char* kt = kbase + (int64_t)page * k_block_bytes + (int64_t)off * 16;
+    const uint32_t kdst = st + (uint32_t)offsetof(StepLds, k) + (uint32_t)wave * 2048u;
+    dma_load16(kt, k_lane_off[0], kdst);
+    dma_load16(kt, k_lane_off[1], kdst + 1024u);
+    const char* vt_ = vbase + (int64_t)page * v_block_bytes + (int64_t)(off >> 4) * v_tile_bytes;
+    const uint32_t vdst = st + (uint32_t)offsetof(StepLds, v) + (uint32_t)wave * 2048u;
+    dma_load16(vt_, v_lane_off[0], vdst);   // head dims 0..63 (lane = dim)
+    dma_load16(vt_, v_lane_off[1], vdst + 1024u);  // head dims 64..127
+    if constexpr (PER_TOKEN) {
+      // lanes 0-15: the K scales of the tile's 16 tokens, lanes 16-31: the V scales
+      if (lane < 32)
+        dma_load4(sc_lane + ((int64_t)page * a.stride_kvscale_b + off),
+                  st + (uint32_t)offsetof(StepLds, sc) + (uint32_t)wave * 128u);
+    }
+  };
+
+  // ---- the first NB-1 steps go out before anything else is set up ----------------------------------------------
+  TilePage pg_next = load_page(wg_start);  // of the next step to fetch
+  int fetch_tok = wg_start;
+#pragma unroll
+  for (int i = 0; i < NB - 1; ++i) {
+    if (i < n_steps) {
+      fetch(i, pg_next);
+      fetch_tok += kStepTokens;
+      pg_next = load_page(fetch_tok);
+    }
+  }
+
+  // ---- buffers of this item ---------------------------------------------------------------------------------
+  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+  char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                     (int64_t)part * a.stride_tmp_p) * 2;
+  const bool direct = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
+  char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+  // ---- per-lane row bookkeeping ---------------------------------------------------------------------------------
+  const bool has_alibi = a.alibi_slopes != nullptr;
+  const int row = row0 + li;
+  const bool row_ok = row < rows_valid;
+  const int t_row = row / G;
+  const int limit = row_ok ? ctx - (qb - 1 - t_row) : 0;  // number of visible keys of this lane's query row
+  float slope2 = 0.f;
+  if (has_alibi && row_ok) slope2 = a.alibi_slopes[h * G + (row - t_row * G)] * kLog2e;
+  const int min_limit = ctx - (qb - 1);
+
+  // ---- query: q * cq = hi + lo in e4m3 (|q * cq| <= 224), the B operand of S^T = K Q^T -------------------
+  float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
+  if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
+    k_tensor_scale = sload_f32(a.key_scale);
+    v_tensor_scale = sload_f32(a.value_scale);
+  }
+  float rscale = a.softmax_scale * k_tensor_scale * kLog2e;
+  if (a.query_quant_mode == PA_QUANT_PER_TENSOR) rscale *= sload_f32(a.query_scale);
+  if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row_ok)
+    rscale *= a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
+  i32x8 qhi, qlo;
+  {
+    const char* q_ptr = (const char*)a.query;
+    const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (row_ok ? row : 0)) * a.stride_q_h;
+    float f[32];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int dim = 64 * (s >> 1) + 16 * kg + 8 * (s & 1);
+      Bf16x8Bits q;
+      if (a.query_dtype == PA_DTYPE_BF16) {
+        q.u = load16(q_ptr + (e0 + dim) * 2);
+      } else {
+        u32x2 raw = *reinterpret_cast<const u32x2*>(q_ptr + e0 + dim);
+        q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
+      }
+      if (!row_ok) q.u = u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f[8 * s + 2 * e] = bf16_bits_to_f32(q.u[e] & 0xffffu);
+        f[8 * s + 2 * e + 1] = __uint_as_float(q.u[e] & 0xffff0000u);
+      }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(f[e]));
+    amax = quad_row_max(amax);
+    const float cq = amax > 0.f ? 224.f / amax : 1.f;
+    rscale *= amax > 0.f ? amax * (1.f / 224.f) : 1.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const float x0 = f[4 * w] * cq, x1 = f[4 * w + 1] * cq, x2 = f[4 * w + 2] * cq, x3 = f[4 * w + 3] * cq;
+      int hi = 0, lo = 0;
+      hi = __builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, hi, false);
+      hi = __builtin_amdgcn_cvt_pk_fp8_f32(x2, x3, hi, true);
+      const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+      const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+      lo = __builtin_amdgcn_cvt_pk_fp8_f32(x0 - b01[0], x1 - b01[1], lo, false);
+      lo = __builtin_amdgcn_cvt_pk_fp8_f32(x2 - b23[0], x3 - b23[1], lo, true);
+      qhi[w] = hi;
+      qlo[w] = lo;
+    }
+  }
+
+  const bool rs_nonneg = __builtin_amdgcn_ballot_w64(rscale < 0.f) == 0;
+  float v_run = 1e-30f;  // per-token V scales: running max of the scales seen so far
+  float m_run = -INFINITY;
+  float l_run = 0.f;
+  f32x4 acc[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- one step of 64 tokens out of LDS: the arithmetic of pa_partition_kernel's FP8 step, one row tile ----
+  auto compute = [&]<bool FULL>(const StepLds& st, int tok0) {
+    f32x4 s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const u32x4 k0 = st.k[j][0][lane], k1 = st.k[j][1][lane];
+      const i32x8 ka = {(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
+      s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      s[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi, s[j], 0, 0, 0, 0, 0, 0);
+      s[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[j], 0, 0, 0, 0, 0, 0);
+    }
+    // P is produced already multiplied by pmul = 256 / v_run (per-token V scales: v_run is the running
+    // maximum of the scales, P then also carries v_scale / v_run <= 1 and the accumulator is kept in units
+    // of v_run): log2(pmul) rides in the exponent's additive term, so it costs nothing per element
+    float vfac = 1.f, log2_pmul = 8.f, inv_pmul = 1.f / 256.f;
+    f32x4 ks_cur[PER_TOKEN ? 4 : 1], vs_cur[PER_TOKEN ? 4 : 1];
+    if constexpr (PER_TOKEN) {
+      float vmx = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ks_cur[j] = *reinterpret_cast<const f32x4*>(&st.sc[j][0][4 * kg]);
+        vs_cur[j] = *reinterpret_cast<const f32x4*>(&st.sc[j][1][4 * kg]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (!FULL) {
+            const int col = tok0 + 16 * j + 4 * kg + r;
+            vs_cur[j][r] = col < ctx ? vs_cur[j][r] : 0.f;
+          }
+          vmx = fmaxf(vmx, vs_cur[j][r]);
+        }
+      }
+      vmx = quad_row_max(vmx);
+      const float v_new = fmaxf(v_run, vmx);
+      vfac = v_new == v_run ? 1.f : v_run * __builtin_amdgcn_rcpf(v_new);
+      log2_pmul = 8.f - __builtin_amdgcn_logf(v_new);
+      inv_pmul = v_new * (1.f / 256.f);
+      v_run = v_new;
+    }
+    // FULL: the row's scale (>= 0 on this path) is applied inside the exponent's fma, and to the maximum once
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = s[j][r];
+        if constexpr (PER_TOKEN) v *= ks_cur[j][r];
+        if constexpr (!FULL) {
+          const int col = tok0 + 16 * j + 4 * kg + r;
+          v = v * rscale + slope2 * (float)(col - ctx + 1);
+          v = col < limit ? v : -INFINITY;
+        }
+        s[j][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    }
+    mx = quad_row_max(mx);
+    if constexpr (FULL) mx *= rscale;
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    m_run = m_new;
+    const float e_add = log2_pmul - m_safe;
+    const float e_mul = FULL ? rscale : 1.f;
+    float psum = 0.f;
+    uint32_t ph[4], pl[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float p0 = fast_exp2(__builtin_fmaf(s[j][0], e_mul, e_add));
+      float p1 = fast_exp2(__builtin_fmaf(s[j][1], e_mul, e_add));
+      float p2 = fast_exp2(__builtin_fmaf(s[j][2], e_mul, e_add));
+      float p3 = fast_exp2(__builtin_fmaf(s[j][3], e_mul, e_add));
+      psum += (p0 + p1) + (p2 + p3);
+      if constexpr (PER_TOKEN) {
+        p0 *= vs_cur[j][0];
+        p1 *= vs_cur[j][1];
+        p2 *= vs_cur[j][2];
+        p3 *= vs_cur[j][3];
+      }
+      int hi = 0, lo = 0;
+      hi = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, hi, false);
+      hi = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, hi, true);
+      const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+      const f32x2 b23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+      lo = __builtin_amdgcn_cvt_pk_fp8_f32(p0 - b01[0], p1 - b01[1], lo, false);
+      lo = __builtin_amdgcn_cvt_pk_fp8_f32(p2 - b23[0], p3 - b23[1], lo, true);
+      ph[j] = (uint32_t)hi;
+      pl[j] = (uint32_t)lo;
+    }
+    l_run = l_run * alpha + psum * inv_pmul;
+    // the accumulator is rescaled only when some row's maximum (or the V scale unit) moved
+    const float alpha_acc = alpha * vfac;
+    if (__builtin_amdgcn_ballot_w64(alpha_acc != 1.f)) {
+#pragma unroll
+      for (int db = 0; db < 8; ++db) acc[db] *= alpha_acc;
+    }
+
+    // lane group kg holds, per tile j, tokens 4kg..4kg+3; the B operand of O^T += V^T P^T wants lane group
+    // kg to hold all 16 tokens of tile kg: a 4x4 transpose over (lane group, register)
+    quad_transpose(ph);
+    quad_transpose(pl);
+    // one 128-deep MFMA per 16 head dims covers head and residual of P at once: its reduction index runs
+    // over (tile kg's 16 tokens with P head, the same 16 tokens with P residual), so the A operand is the V
+    // bytes twice -- read from LDS twice, which costs no VALU slot
+    const i32x8 pb = {(int)ph[0], (int)ph[1], (int)ph[2], (int)ph[3], (int)pl[0], (int)pl[1], (int)pl[2], (int)pl[3]};
+    int nvalid = 16;
+    if constexpr (!FULL) {
+      // V bytes of tokens at or beyond ctx are zeroed (stale cache contents may decode to NaN)
+      nvalid = ctx - (tok0 + 16 * kg);
+      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+    }
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const u32x4* vp = &st.v[kg][16 * db + li];
+      typedef const volatile __attribute__((address_space(3))) u32x4* LdsVec;
+      u32x4 v0 = *vp;
+      u32x4 v1 = *(LdsVec)vp;  // a second LDS read, not a register copy
+      if constexpr (!FULL) {
+        v0 = keep_first_bytes(v0, nvalid);
+        v1 = keep_first_bytes(v1, nvalid);
+      }
+      const i32x8 va = {(int)v0[0], (int)v0[1], (int)v0[2], (int)v0[3], (int)v1[0], (int)v1[1], (int)v1[2], (int)v1[3]};
+      acc[db] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, pb, acc[db], 0, 0, 0, 0, 0, 0);
+    }
+  };
+
+  // ---- main loop ---------------------------------------------------------------------------------------------
+  int n_full = has_alibi ? 0 : (min_limit - wg_start) / kStepTokens;  // leading steps that need no masking
+  n_full = n_full < 0 ? 0 : n_full;
+  int tok0 = wg_start;
+  int slot = 0;             // ring slot of step s
+  int fetch_slot = NB - 1;  // ring slot the next fetch goes to
+  int s = 0;
+  // what every wave does at the head of step s, whether it has rows to compute or not
+  auto enter_step = [&]() {
+    // step s has landed once at most the loads of the steps after it are outstanding
+    const int after = n_steps - 1 - s;
+    if (after >= NB - 2)
+      dma_wait<(NB - 2) * kLoadsPerStep>();
+    else if (NB > 3 && after == 1)
+      dma_wait<kLoadsPerStep>();
+    else
+      dma_wait<0>();
+    // everybody's quarter of step s is in LDS, and everybody is done reading step s-1, whose slot is refilled now
+    __syncthreads();
+    if (s + NB - 1 < n_steps) {
+      fetch(fetch_slot, pg_next);
+      fetch_tok += kStepTokens;
+      pg_next = load_page(fetch_tok);
+    }
+  };
+  auto leave_step = [&]() {
+    ++s;
+    tok0 += kStepTokens;
+    slot = slot + 1 == NB ? 0 : slot + 1;
+    fetch_slot = fetch_slot + 1 == NB ? 0 : fetch_slot + 1;
+  };
+  // Three loops, each with one variant of the step (one loop with a choice inside would make the compiler
+  // copy the whole accumulator state where the variants join, every step).  The waves of a workgroup may be
+  // in different loops: all of them pass the same number of barriers.
+  if (has_rows) {
+    const int n_fast = rs_nonneg ? (n_full < n_steps ? n_full : n_steps) : 0;
+    while (s < n_fast) {
+      enter_step();
+      compute.template operator()<true>(stage[slot], tok0);
+      leave_step();
+    }
+    while (s < n_steps) {
+      enter_step();
+      compute.template operator()<false>(stage[slot], tok0);
+      leave_step();
+    }
+  } else {
+    while (s < n_steps) {
+      enter_step();
+      leave_step();
+    }
+  }
+  __syncthreads();  // the stage buffers are free
+
+  // ---- epilogue: every wave writes its own row tile -----------------------------------------------------------
+  if (!has_rows) {
+    // a tile of padding rows only (a ragged batch): the rows read as "no visible key"
+    for (int r = row0 + kg; r < row0 + 16 && r < Ge; r += 4) {
+      if (li == 0) {
+        a.max_logits[es_off + r] = -INFINITY;
+        a.exp_sums[es_off + r] = 0.f;
+      }
+      *reinterpret_cast<u32x4*>(tmp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
+      if (direct) *reinterpret_cast<u32x4*>(outp + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
+    }
+    return;
+  }
+  float l_tot = quad_row_sum(l_run);
+  if (!row_ok) {
+    l_tot = 0.f;
+    m_run = -INFINITY;
+  }
+  const float acc_unit = (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f);
+  const float inv = l_tot > 0.f ? v_tensor_scale * acc_unit / l_tot : 0.f;
+  if (row < Ge && kg == 0) {
+    a.max_logits[es_off + row] = m_run * (1.0f / kLog2e);
+    a.exp_sums[es_off + row] = l_tot;
+  }
+  char* olds = reinterpret_cast<char*>(&stage[0]) + wave * (16 * kORowBytes);
+  store_partial_tile(olds, acc, inv, tmp + (int64_t)row0 * a.stride_tmp_g * 2, a.stride_tmp_g * 2,
+                     direct ? outp + (int64_t)row0 * a.stride_out_h * 2 : nullptr, a.stride_out_h * 2, Ge - row0, lane);
+}
+
+}  // namespace
+
+#endif  // PA_PARTITION_SHARED_KERNEL_H_
