@@ -43,14 +43,15 @@ def _run(wl, dev, *, partition_size=256, alibi=None, transposed=False, **kw):
 def _oracle(wl, alibi=None, seq_ids=None):
     return O.paged_attention_decode_oracle(
         wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
-        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, alibi, seq_ids)
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, alibi, seq_ids, q_max=wl.q_len)
 
 
 def _check_stages(wl, res, partition_size, alibi=None):
     P = res["maximum_logits"].shape[2]
     ml, es, to = O.partition_stage(
         wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
-        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, alibi, partition_size, P)
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, alibi, partition_size, P,
+        q_max=wl.q_len)
     gml, ges = res["maximum_logits"].cpu(), res["exponential_sums"].cpu()
     gto = res["temporary_output"].float().cpu()
     fin = torch.isfinite(ml)
@@ -362,3 +363,44 @@ def test_scaled_down_benchmark_configs(cuda, name, batch, ctx_scale):
     print(f"config={wl.name} ctx={wl.context_lens.tolist()}", flush=True)
     out, res = _run(wl, cuda, partition_size=None)
     torch.testing.assert_close(out.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+
+
+def _random_case(seed):
+    """One seeded draw over the whole supported parameter space of the op."""
+    gen = torch.Generator().manual_seed(1000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=gen))]
+
+    kv_dtype = pick(["fp8", "fp8", "fp8", "bf16"])
+    block_size = pick([16, 16, 64, 1024])
+    q_len = pick([1, 1, 2, 3, 4])
+    group = pick([g for g in (1, 2, 3, 4, 5, 7, 8, 10, 12, 16, 16, 16) if g * q_len <= 64 and (kv_dtype == "fp8" or g * q_len <= 16)])
+    hkv = pick([1, 2, 3])
+    batch = pick([1, 2, 3, 5])
+    max_ctx = pick([40, 300, 1100, 2600])
+    ctx = torch.randint(q_len, max_ctx + 1, (batch,), generator=gen, dtype=torch.int32)
+    kw = dict(batch=batch, num_q_heads=group * hkv, num_kv_heads=hkv, context_lens=ctx, q_len=q_len,
+              block_size=block_size, kv_dtype=kv_dtype, seed=seed,
+              scale_mode="none" if kv_dtype == "bf16" else pick(["tensor", "token"]),
+              transposed_v=pick([False, True]))
+    if q_len > 1 and pick([False, True]):
+        kw["q_lens"] = torch.randint(1, q_len + 1, (batch,), generator=gen, dtype=torch.int32)
+    ps = pick([256, 512, 768, 2048, None])
+    alibi = pick([False, False, True])
+    return kw, ps, alibi
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_seeded_random_sweep(cuda, seed):
+    """Random shapes, layouts, scale modes, partition sizes and ALiBi: the HIP path against the oracle end to
+    end and stage by stage."""
+    kw, ps, alibi = _random_case(seed)
+    print(f"seed={seed} ps={ps} alibi={alibi} " + " ".join(f"{k}={v.tolist() if torch.is_tensor(v) else v}" for k, v in kw.items()),
+          flush=True)
+    wl = _make(**kw)
+    slopes = torch.linspace(0.02, 0.4, wl.num_q_heads, dtype=torch.float32) if alibi else None
+    out, res = _run(wl, cuda, partition_size=ps, alibi=slopes)
+    assert not torch.isnan(out.float()).any()
+    torch.testing.assert_close(out.float(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
+    _check_stages(wl, res, res["partition_size"], slopes)
