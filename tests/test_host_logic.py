@@ -165,3 +165,22 @@ def test_per_token_quantised_cache_layout():
     assert float((vback - vtok).abs().max()) <= float(vtok.abs().max()) * 2.0 ** -4
     kq2, ks2, vq2, vs2 = L.quantize_kv_cache_per_tensor(kc, vc)
     assert kq2.shape == kq.shape and ks2.dim() == 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU per box: bench.py --gpus N with N > 1 must say so and exit instead of measuring anything."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                         text=True, timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in (res.stdout + res.stderr)
+
+
+def test_graft_entry_points_exist():
+    import __graft_entry__ as g
+
+    assert callable(g.build) and callable(g.smoke)
