@@ -9,12 +9,18 @@ namespace {
 // ---------------------------------------------------------------------------------------------
 // Partition kernel for more than 16 query rows per kv head (large GQA groups, MTP) over an FP8 cache.
 // The up to four 16-row query tiles of one (sequence, kv head, partition) are the four waves of ONE
-// workgroup and share a single pass over the pages.  Of every 64-token step each wave fetches a quarter
-// (K tile `wave`, V head-dim blocks 2*wave and 2*wave+1) into registers and parks it in LDS in exactly the
-// per-lane operand order of the MFMAs; after a workgroup barrier every wave reads the whole step back
-// with lane-contiguous 16-byte LDS reads.  Two LDS buffers: step s+1 travels from HBM while step s is multiplied,
-// one barrier per step.  Against one workgroup per row tile this reads every page once instead of once per
-// tile (the repeats hit the L2, but each costs a full trip through the vector memory path).
+// workgroup and share a single pass over the pages.  Of every 64-token step wave w fetches tile w (K 2 KiB,
+// V 2 KiB, the tile's per-token scales) straight from global memory into LDS (global_load_lds, no
+// registers), laid out in exactly the per-lane operand order of the MFMAs; after a workgroup barrier every
+// wave reads the whole step back with lane-contiguous 16-byte LDS reads and runs the step's arithmetic for
+// its own 16 rows.  LDS holds a ring of NB steps: NB-1 travel from HBM while one is multiplied; one barrier
+// per step.  Against one workgroup per row tile this reads every page once instead of once per tile (the
+// repeats hit the L2, but each costs a full trip through the vector memory path) and sets an item up once.
+//
+// The asynchronous loads are invisible to the compiler, which therefore inserts no waits for them: the wave
+// that issued them waits with dma_wait<n>() before the barrier.  Nothing inside the step loop may use
+// scratch memory (a spill, an indexed private array): the compiler would wait for such a load with
+// vmcnt(0) and drain the ring.
 // ---------------------------------------------------------------------------------------------
 struct StepLds {
   u32x4 k[4][2][64];  // [tile][load][lane]: the K operand of a tile as its two loads deliver it
@@ -50,7 +56,11 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int n_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
   const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
   const int rows_valid = qb * G;
-  const int row0 = 16 * wave;               // this wave's query tile
+  // The waves of a workgroup are spread over the CU's four SIMDs, and in a ragged batch tile 0 is always busy
+  // while tile 3 rarely is: which wave computes which tile rotates from workgroup to workgroup, so that no
+  // SIMD collects the busy tiles of every resident workgroup (worth ~3 % on ragged query lengths).  Which
+  // wave fetches which quarter of a step does not rotate.
+  const int row0 = 16 * ((wave + b + h + part) & 3);  // this wave's query tile
   const bool has_rows = row0 < rows_valid;  // else the wave only helps to fetch
 
   // ---- cache addressing ----------------------------------------------------------------------------------
