@@ -21,11 +21,16 @@
 extern "C" {
 #endif
 
-#define PA_DECODE_ABI_VERSION 2
-/* Size of the optional device workspace.  It holds a work-item counter: with it, ragged batches are launched
- * as a resident grid that pulls live (sequence, partition, row tile, head) items from the counter instead
- * of one workgroup per possible item.  It must be zero before the first call; every call leaves it zero.
- * Calls that may overlap on the GPU need a workspace each. */
+#define PA_DECODE_ABI_VERSION 3
+/* Smallest useful size of the optional device workspace.  Its first 64 bytes hold a work-item counter: with
+ * it, batches with per-sequence query lengths are launched as a resident grid that pulls live (sequence,
+ * partition, row tile, head) items from the counter instead of one workgroup per possible item.  These 64
+ * bytes must be zero before the first call; every call leaves them zero.  A workspace of
+ * pa_decode_workspace_bytes() bytes also has room for the work-item list of the sorted dispatch: in launches of
+ * several rounds of workgroups a small planning kernel lists the live (sequence, partition) items, whole
+ * partitions first and the sequences' last, partial partitions by decreasing length, and the partition kernel
+ * takes its items from the list (longest-first keeps the end of a ragged batch's launch busy).  The list is
+ * rewritten by every call.  Calls that may overlap on the GPU need a workspace each. */
 #define PA_DECODE_WORKSPACE_BYTES 64
 
 /* element types */
@@ -67,7 +72,7 @@ enum {
  */
 typedef struct PaDecodeArgs {
   uint32_t struct_size; /* = sizeof(PaDecodeArgs) */
-  int32_t reserved0;
+  int32_t reserved0;     /* 0 */
 
   void* output;
   const void* query;
@@ -84,7 +89,7 @@ typedef struct PaDecodeArgs {
   float* exp_sums;
   float* max_logits;
   void* tmp_output;
-  int32_t* workspace;         /* optional, >= PA_DECODE_WORKSPACE_BYTES, zero on entry; left zero on return */
+  int32_t* workspace;         /* optional, workspace_bytes long; first 64 bytes zero on entry, left zero on return */
 
   int32_t num_seqs;
   int32_t num_kv_heads;
@@ -110,6 +115,7 @@ typedef struct PaDecodeArgs {
   int64_t stride_tmp_s, stride_tmp_h, stride_tmp_p, stride_tmp_g;
   int64_t stride_qscale_s;                        /* per-token query scale: stride of dim 0 */
   int64_t stride_kvscale_b, stride_kvscale_h;     /* per-token kv scales: block, kv head */
+  int64_t workspace_bytes;                        /* size of workspace (>= PA_DECODE_WORKSPACE_BYTES), 0 without one */
 } PaDecodeArgs;
 
 /* Library / ABI identification. */
@@ -118,6 +124,8 @@ uint32_t pa_decode_args_size(void);
 const char* pa_decode_error_string(int code);
 /* hipError_t of the last failed launch on the calling thread (0 if none). */
 int pa_decode_last_hip_error(void);
+/* Workspace size that enables every launch mode for a batch of this shape (see PA_DECODE_WORKSPACE_BYTES). */
+int64_t pa_decode_workspace_bytes(int32_t num_seqs, int32_t max_num_partitions);
 
 /*
  * Launch-time tuning layer; replaces the constants and the 15 lines of kernel selection in

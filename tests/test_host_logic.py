@@ -51,6 +51,13 @@ def test_struct_layout_and_version(pa_lib):
     assert C.sizeof(_cabi.PaKvWriteArgs) == 8 + 7 * 8 + 8 + 6 * 4 + 10 * 8
 
 
+def test_workspace_size_rule(pa_lib):
+    # 64 bytes of counters + one (sequence, partition) pair of int32 per possible item
+    assert pa_lib.pa_decode_workspace_bytes(256, 8) == 64 + 8 * 256 * 8
+    assert pa_lib.pa_decode_workspace_bytes(1, 1) == 72
+    assert pa_lib.pa_decode_workspace_bytes(0, 4) == _cabi.PA_DECODE_WORKSPACE_BYTES
+
+
 def test_error_strings_and_null_arguments(pa_lib):
     assert pa_lib.pa_decode_error_string(0) == b"ok"
     for code in range(-6, 0):

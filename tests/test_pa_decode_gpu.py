@@ -322,6 +322,37 @@ def test_many_rows_take_the_four_rows_per_wave_reduce(cuda, with_sinks):
     torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("group,q_len,scale_mode", [(8, 1, "tensor"), (16, 3, "token"), (4, 2, "tensor")])
+def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
+    """Launches with several rounds of workgroups take their (sequence, partition) items from the planning
+    kernel's list (whole partitions first, last partitions by decreasing length).  The result must be the one the
+    plain grid order gives, bit for bit, with a minimal workspace (no list) and with none of the counters left
+    behind; one-token sequences and exact multiples of the partition size are in the batch."""
+    import triton_op_amd as T
+
+    gen = torch.Generator().manual_seed(21)
+    batch = 96
+    ctx = torch.randint(1, 2600, (batch,), generator=gen, dtype=torch.int32)
+    ctx[:5] = torch.tensor([512, 256, 2560, 1, 255], dtype=torch.int32)
+    ctx = torch.clamp(ctx, min=q_len)
+    wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, scale_mode=scale_mode)
+    g = wl.to(cuda)
+    outs = []
+    for ws_bytes in (None, 64):  # None: the entry point sizes the workspace for the item list; 64: counters only
+        ws = None if ws_bytes is None else torch.zeros(ws_bytes // 4, dtype=torch.int32, device=cuda)
+        out = torch.full_like(g.query, float("nan"))
+        plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                             g.softmax_scale, q_len, g.max_context_len, torch.bfloat16, None, g.key_scale,
+                             g.value_scale, partition_size=256, workspace=ws)
+        assert plan.args.max_num_partitions * batch * 8 > 4096  # far more workgroups than the GPU holds
+        plan.run()
+        plan.run()  # the list is rebuilt by every call
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+
+
 @pytest.mark.parametrize("name", ["fp8_g8", "fp8_token_g16_q4"])
 def test_negative_softmax_scale(cuda, name):
     """A negative scale turns the row maximum of the raw logits into the minimum of the scaled ones: the

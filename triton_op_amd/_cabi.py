@@ -12,7 +12,7 @@ import threading
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
-PA_DECODE_ABI_VERSION = 2
+PA_DECODE_ABI_VERSION = 3
 PA_DECODE_WORKSPACE_BYTES = 64
 PA_DTYPE_BF16, PA_DTYPE_FP8_E4M3FN = 0, 1
 PA_QUANT_NONE, PA_QUANT_PER_TENSOR, PA_QUANT_PER_TOKEN = -1, 0, 1
@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "pa_decode_args_size",
     "pa_decode_error_string",
     "pa_decode_last_hip_error",
+    "pa_decode_workspace_bytes",
     "pa_decode_select_partition_size",
     "pa_decode_partition",
     "pa_decode_reduce",
@@ -49,7 +50,7 @@ class PaDecodeArgs(C.Structure):
             "stride_k_b", "stride_k_h", "stride_k_c", "stride_v_b", "stride_v_h", "stride_v_2",
             "stride_bt_s", "stride_es_s", "stride_es_h", "stride_es_p",
             "stride_tmp_s", "stride_tmp_h", "stride_tmp_p", "stride_tmp_g",
-            "stride_qscale_s", "stride_kvscale_b", "stride_kvscale_h")]
+            "stride_qscale_s", "stride_kvscale_b", "stride_kvscale_h", "workspace_bytes")]
     )
 
 
@@ -91,6 +92,8 @@ def load_library(path: str = None) -> C.CDLL:
         lib.pa_decode_error_string.restype = C.c_char_p
         lib.pa_decode_error_string.argtypes = [C.c_int]
         lib.pa_decode_last_hip_error.restype = C.c_int
+        lib.pa_decode_workspace_bytes.restype = C.c_int64
+        lib.pa_decode_workspace_bytes.argtypes = [C.c_int32, C.c_int32]
         lib.pa_decode_select_partition_size.restype = C.c_int
         lib.pa_decode_select_partition_size.argtypes = [C.c_int32] * 6
         for name in ("pa_decode_partition", "pa_decode_reduce", "pa_decode"):

@@ -16,6 +16,7 @@
 #include "pa_common.h"
 #include "pa_partition_kernel.h"
 #include "pa_partition_shared_kernel.h"
+#include "pa_plan_kernel.h"
 #include "pa_reduce_kernel.h"
 
 namespace {
@@ -42,6 +43,7 @@ int check_common(const PaDecodeArgs* a) {
       a->max_num_partitions <= 0)
     return PA_ERR_BAD_SHAPE;
   if (a->partition_size <= 0 || a->partition_size % 256) return PA_ERR_BAD_SHAPE;
+  if (a->workspace ? a->workspace_bytes < PA_DECODE_WORKSPACE_BYTES : a->workspace_bytes != 0) return PA_ERR_BAD_SHAPE;
   if (a->head_size != kHeadSize) return PA_ERR_UNSUPPORTED;
   if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;  // the reference's limit
   return PA_OK;
@@ -69,6 +71,34 @@ bool use_queue(const PaDecodeArgs& a) {
   return !off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr;
 }
 
+// Bytes of workspace the sorted dispatch needs: the header and one (sequence, partition) pair per possible item.
+long long plan_workspace_bytes(int num_seqs, int max_num_partitions) {
+  return 4LL * kPlanHeaderWords + 8LL * num_seqs * max_num_partitions;
+}
+
+// The sorted dispatch pays a small extra kernel, and ordering only matters when workgroups are handed out in
+// several rounds: it is used when the launch has more than twice as many workgroups as the GPU holds at once
+// and the caller's workspace has room for the list.  PA_DECODE_SORTED=0 switches it off, =1 drops the size rule.
+bool use_sorted_items(const PaDecodeArgs& a, long long blocks, int workgroups_per_cu) {
+  static const int mode = [] {
+    const char* e = getenv("PA_DECODE_SORTED");
+    return e ? atoi(e) : -1;
+  }();
+  if (mode == 0 || a.workspace == nullptr || a.num_seqs > kPlanMaxSeqs) return false;
+  if (a.workspace_bytes < plan_workspace_bytes(a.num_seqs, a.max_num_partitions)) return false;
+  return mode == 1 || blocks > 2LL * device_num_cus() * workgroups_per_cu;
+}
+
+int launch_plan(const PaDecodeArgs& a, hipStream_t stream) {
+  hipLaunchKernelGGL(pa_plan_kernel, dim3(1), dim3(1024), 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return PA_OK;
+}
+
 template <int NT, int KVT, bool PT, bool BS16, int W>
 int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   constexpr int OCC = NT == 1 ? 2 : 1;
@@ -79,10 +109,21 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
   if (use_queue(a)) {
     long long resident = (long long)device_num_cus() * 4 * OCC / W;
     resident = resident < blocks ? resident : blocks;
+    PaDecodeArgs k = a;
+    k.reserved0 = 0;
     hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)resident),
-                       dim3(64 * W), 0, stream, a);
-  } else
-  hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)blocks), dim3(64 * W), 0, stream, a);
+                       dim3(64 * W), 0, stream, k);
+  } else {
+    PaDecodeArgs k = a;
+    k.reserved0 = 0;
+    if (use_sorted_items(a, blocks, 4 * OCC / W)) {
+      const int rc = launch_plan(a, stream);
+      if (rc) return rc;
+      k.reserved0 = kFlagSortedItems;
+    }
+    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)blocks), dim3(64 * W), 0,
+                       stream, k);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
@@ -135,10 +176,18 @@ int launch_partition_shared(const PaDecodeArgs& a, hipStream_t stream) {
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
   // ring depth / waves per SIMD: without per-token scales the kernel fits 128 registers, and a fourth workgroup
   // per CU is worth more than a deeper ring (measured); with them it needs about 140
+  constexpr int kWorkgroupsPerCu = PT ? 3 : 4;
+  PaDecodeArgs k = a;
+  k.reserved0 = 0;
+  if (use_sorted_items(a, blocks, kWorkgroupsPerCu)) {
+    const int rc = launch_plan(a, stream);
+    if (rc) return rc;
+    k.reserved0 = kFlagSortedItems;
+  }
   if constexpr (PT)
-    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, k);
   else
-    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, k);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error = (int)e;
@@ -200,6 +249,11 @@ extern "C" {
 int pa_decode_abi_version(void) { return PA_DECODE_ABI_VERSION; }
 uint32_t pa_decode_args_size(void) { return (uint32_t)sizeof(PaDecodeArgs); }
 int pa_decode_last_hip_error(void) { return g_last_hip_error; }
+
+int64_t pa_decode_workspace_bytes(int32_t num_seqs, int32_t max_num_partitions) {
+  if (num_seqs <= 0 || max_num_partitions <= 0) return PA_DECODE_WORKSPACE_BYTES;
+  return plan_workspace_bytes(num_seqs, max_num_partitions);
+}
 
 const char* pa_decode_error_string(int code) {
   switch (code) {

@@ -150,8 +150,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     const long long wid = blockIdx.x;
     h = (int)(wid % Hkv);
     rt = (int)((wid / Hkv) % RT);
-    b = (int)((wid / ((long long)Hkv * RT)) % a.num_seqs);
-    part = (int)(wid / ((long long)Hkv * RT * a.num_seqs));
+    const long long item = wid / ((long long)Hkv * RT);
+    if (a.reserved0 & kFlagSortedItems) {
+      // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
+      if (item >= sload_i32(a.workspace + 2)) return;
+      b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);
+      part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1);
+    } else {
+      b = (int)(item % a.num_seqs);
+      part = (int)(item / a.num_seqs);
+    }
   }
   const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
   do {  // the body of one item; `break` leaves it

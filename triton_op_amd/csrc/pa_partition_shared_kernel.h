@@ -46,8 +46,17 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int Ge = a.q_len * G;
   const long long wid = blockIdx.x;
   const int h = (int)(wid % Hkv);
-  const int b = (int)((wid / Hkv) % a.num_seqs);
-  const int part = (int)(wid / ((long long)Hkv * a.num_seqs));
+  const long long item = wid / Hkv;
+  int b, part;
+  if (a.reserved0 & kFlagSortedItems) {
+    // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
+    if (item >= sload_i32(a.workspace + 2)) return;
+    b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);
+    part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1);
+  } else {
+    b = (int)(item % a.num_seqs);
+    part = (int)(item / a.num_seqs);
+  }
 
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;

@@ -16,8 +16,10 @@ pa_decode_triton.py:523-685.  Differences, all additive:
 * `sinks` gives an attention-sink logit per query row ([num_kv_heads * query_group_size], as the reference's
   Gluon reduce kernel indexes it, pa_decode_triton_gluon_fp8.py:1118-1123): exp(sink - max) joins the softmax
   denominator;
-* `workspace` is a zeroed int32 tensor of 64 bytes holding a work-item counter for ragged batches (one is
-  allocated per call/plan when it is not given; calls that may overlap on the GPU need one each).
+* `workspace` is an int32 tensor of at least 64 bytes whose first 64 bytes are zero (a work-item counter for
+  ragged batches); with `pa_decode_workspace_bytes(num_seqs, partitions)` bytes it also has room for the item
+  list of the sorted dispatch.  One is allocated per call/plan when it is not given; calls that may overlap on
+  the GPU need one each.
 
 There is no eager/torch implementation behind this function: without the HIP library it raises.
 """
@@ -286,13 +288,16 @@ def plan_decode(
     a.alibi_slopes = _ptr(alibi_slopes)
     a.sinks = _ptr(sinks)
     a.exp_sums, a.max_logits, a.tmp_output = exp_sums.data_ptr(), max_logits.data_ptr(), tmp_output.data_ptr()
-    # zeroed work-item counter for ragged batches; the kernels leave it zero, so the plan can be replayed
+    # zeroed work-item counter for ragged batches (the kernels leave it zero, so the plan can be replayed) plus
+    # room for the item list of the sorted dispatch
     if workspace is None:
-        workspace = torch.zeros(_cabi.PA_DECODE_WORKSPACE_BYTES // 4, dtype=torch.int32, device=dev)
+        need = int(_cabi.load_library().pa_decode_workspace_bytes(num_seqs, max_parts))
+        workspace = torch.zeros((need + 3) // 4, dtype=torch.int32, device=dev)
     elif workspace.dtype != torch.int32 or workspace.numel() * 4 < _cabi.PA_DECODE_WORKSPACE_BYTES or \
             not workspace.is_contiguous() or workspace.device != dev:
         raise ValueError(f"workspace must be a contiguous int32 tensor of >= {_cabi.PA_DECODE_WORKSPACE_BYTES} bytes on {dev}")
     a.workspace = workspace.data_ptr()
+    a.workspace_bytes = workspace.numel() * 4
     a.num_seqs, a.num_kv_heads, a.group_size, a.q_len = num_seqs, num_kv_heads, group, q_len
     a.head_size, a.block_size = head_size, block_size
     a.max_num_partitions, a.partition_size = max_parts, partition_size
