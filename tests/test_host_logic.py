@@ -76,8 +76,8 @@ def test_partition_size_choices():
     assert f(64, 8, 8, 4096, 16, 256) == 4096      # c2: one partition, four waves per workgroup, no reduce
     assert f(4, 8, 8, 131072, 16, 256) == 8192     # c4: 16 partitions x 32 (sequence, head) pairs x 4 waves
     assert f(128, 8, 16, 32768, 1024, 256) == 8192  # c3
-    assert f(256, 8, 64, 65536, 16, 256) == 4096   # c5: 64 rows = 4 row tiles sharing one workgroup's page stream
-    assert f(4, 8, 32, 131072, 16, 256) == 4096    # few long sequences, 2 row tiles: 32 partitions fill the GPU
+    assert f(256, 8, 64, 65536, 16, 256) == 8192   # c5: 64 rows = 4 row tiles sharing one workgroup's page stream
+    assert f(4, 8, 32, 131072, 16, 256) == 5632    # few long sequences, 2 row tiles: 24 partitions fill the GPU
     assert f(4, 1, 8, 1024, 16, 256) == 256        # c1: tiny, the finest split
     for args in [(1, 1, 1, 1, 16, 256), (3, 5, 7, 100000, 64, 304), (1000, 8, 16, 300, 16, 64)]:
         ps = f(*args)

@@ -281,15 +281,16 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   const int total_tiles = (rows_per_group + 15) / 16;
   if (use_shared_stream(PA_DTYPE_FP8_E4M3FN, rows_per_group)) {
     // All row tiles of a kv head in one workgroup that walks its partition alone: three workgroups fit a CU, and
-    // no workgroup gets more than 4096 tokens (measured on a ragged batch: 3072-4096 is the flat optimum, 8192
-    // costs 7 % in balance, 1024 costs 8 % in partials and merge).
+    // no workgroup gets more than 8192 tokens (measured on a ragged batch with the sorted dispatch: 6144-12288
+    // is the flat optimum, 2048 costs 12 % in partials and merge, 32768 costs 45 % in balance; without the sorted
+    // dispatch the optimum is 3072-4096 and 8192 costs 3 % more).
     const long long slots = (long long)num_cus * 3;
     const long long items = (long long)num_seqs * num_kv_heads;
     for (int parts = 1;; ++parts) {
       int ps = (max_context_len + parts - 1) / parts;
       ps = (ps + 255) / 256 * 256;
       if (ps <= 256) return 256;
-      if (ps <= 4096 && items * parts >= slots) return ps;
+      if (ps <= 8192 && items * parts >= slots) return ps;
     }
   }
   const int nt = tiles_per_workgroup(total_tiles);
