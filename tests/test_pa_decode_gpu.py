@@ -353,6 +353,59 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("case", ["queue", "sorted", "plain"])
+def test_graph_capture_and_replay(cuda, case):
+    """A decode plan allocates nothing and only launches kernels on the given stream, so it can be captured
+    in a HIP graph: every replay (with eager work and synchronisations in between, and with new inputs written
+    into the captured tensors) must reproduce the eager result bit for bit.  Covers the launch modes that keep
+    state in the workspace: the work queue (its counters return to zero) and the sorted dispatch (its list is
+    rebuilt by every call)."""
+    import triton_op_amd as T
+
+    gen = torch.Generator().manual_seed(31)
+    if case == "queue":  # bf16 cache, 32 query rows, ragged query lengths: the queued launch
+        kw = dict(batch=6, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000, 17, 700, 256), q_len=4,
+                  q_lens=_ctx(1, 4, 2, 3, 4, 1), kv_dtype="bf16", scale_mode="none")
+    elif case == "sorted":  # several rounds of workgroups: the planning kernel runs inside the graph
+        kw = dict(batch=96, num_q_heads=32, num_kv_heads=8, q_len=2,
+                  context_lens=torch.randint(2, 2600, (96,), generator=gen, dtype=torch.int32))
+    else:
+        kw = dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000))
+    wl = _make(**kw)
+    g = wl.to(cuda)
+    out = torch.full_like(g.query, float("nan"))
+    plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                         g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                         partition_size=256, query_lens=g.q_lens)
+    plan.run()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    torch.testing.assert_close(eager.float().cpu(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        plan.run(stream=side.cuda_stream)  # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            plan.run(stream=side.cuda_stream)
+    torch.cuda.synchronize()
+    q2 = (g.query.float() * 0.5).to(g.query.dtype)
+    for i in range(3):
+        out.fill_(float("nan"))
+        (g.key_cache.float()[:1] * 1.0).sum().item()  # unrelated eager work and a host sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {i}"
+    # new inputs through the captured tensors: the graph computes the new result
+    g.query.copy_(q2)
+    graph.replay()
+    torch.cuda.synchronize()
+    wl2 = type(wl)(**{**wl.__dict__, "query": q2.cpu()})
+    torch.testing.assert_close(out.float().cpu(), _oracle(wl2).float(), atol=ATOL, rtol=RTOL)
+
+
 @pytest.mark.parametrize("name", ["fp8_g8", "fp8_token_g16_q4"])
 def test_negative_softmax_scale(cuda, name):
     """A negative scale turns the row maximum of the raw logits into the minimum of the scaled ones: the
