@@ -33,6 +33,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_shared_kernel(const PaDecodeArgs a) {
   __shared__ __attribute__((aligned(16))) StepLds stage[NB];  // ring of steps: NB-1 in flight, one being read
   static_assert(sizeof(StepLds) * NB >= 4 * 16 * kORowBytes, "the output tiles reuse the stage buffers");
+  static_assert(sizeof(StepLds) * NB <= 65536, "the LDS address of an asynchronous load travels in 16 bits of M0");
   constexpr int kLoadsPerStep = PER_TOKEN ? 5 : 4;  // vector memory operations one wave issues per step
 
   const int lane = threadIdx.x & 63;
