@@ -78,7 +78,9 @@ def test_partition_size_choices():
     assert f(128, 8, 16, 32768, 1024, 256) == 8192  # c3
     assert f(256, 8, 64, 65536, 16, 256) == 8192   # c5: 64 rows = 4 row tiles sharing one workgroup's page stream
     assert f(4, 8, 32, 131072, 16, 256) == 5632    # few long sequences, 2 row tiles: 24 partitions fill the GPU
-    assert f(4, 1, 8, 1024, 16, 256) == 256        # c1: tiny, the finest split
+    assert f(4, 1, 8, 1024, 16, 256) == 1024       # c1: tiny; one partition, no second kernel
+    assert f(48, 8, 8, 4096, 16, 256) == 4096      # three quarters of the wave slots filled: still one partition
+    assert f(4, 8, 8, 4096, 16, 256) == 1024       # 32 rows only: four partitions each
     for args in [(1, 1, 1, 1, 16, 256), (3, 5, 7, 100000, 64, 304), (1000, 8, 16, 300, 16, 64)]:
         ps = f(*args)
         assert ps >= 256 and ps % 256 == 0

@@ -273,11 +273,6 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   (void)block_size;
   if (num_seqs <= 0 || num_kv_heads <= 0 || max_context_len <= 0 || rows_per_group <= 0) return PA_ERR_BAD_SHAPE;
   if (num_cus <= 0) num_cus = device_num_cus();
-  // The fewest partitions per sequence that still give every wave slot of the GPU a wave: each extra
-  // partition costs a (rows x 128) bf16 partial written and read back plus the merge, and a single
-  // partition needs no second kernel at all.  A workgroup (one 16-row query tile) splits its partition over
-  // up to 4 waves (at least 256 tokens each); no wave is given more than 2048 tokens, which keeps ragged
-  // batches balanced.
   const int total_tiles = (rows_per_group + 15) / 16;
   if (use_shared_stream(PA_DTYPE_FP8_E4M3FN, rows_per_group)) {
     // All row tiles of a kv head in one workgroup that walks its partition alone: three workgroups fit a CU, and
@@ -293,17 +288,38 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
       if (ps <= 8192 && items * parts >= slots) return ps;
     }
   }
+  // One workgroup per 16-row query tile, up to 4 waves (at least 256 tokens each) per workgroup, no wave with
+  // more than 2048 tokens (which keeps ragged batches balanced).  The number of partitions per sequence is the
+  // one a small cost model likes best (times in microseconds on this GPU):
+  //   a wave's 64-token step takes the longer of 1.4 us (one wave alone: a 16 KiB step per HBM round trip) and
+  //   its share of the HBM stream when `waves` of them run at once, 16 KiB * waves / 6.0 TB/s (more waves than
+  //   the GPU holds simply queue: the same formula);
+  //   splitting a sequence costs the second kernel (7 us) and its partials (written, read back: 2 ns per
+  //   16-row tile and partition).
+  // Few rows and long contexts want many partitions; 256 or more rows want one, even if that leaves a quarter
+  // of the wave slots empty (measured at 48 sequences x 8 kv heads x 4096 tokens: 78 us against 87 us for two).
   const int nt = tiles_per_workgroup(total_tiles);
   const int cap_w = nt <= 1 ? 4 : 2;
-  const long long slots = (long long)num_cus * 4 * (nt <= 1 ? 2 : 1);
-  const long long rows = (long long)num_seqs * num_kv_heads * ((total_tiles + nt - 1) / nt);
+  const double rows = (double)num_seqs * num_kv_heads * ((total_tiles + nt - 1) / nt);
+  const double step_us_per_wave = 16384.0 / 6.0e6;  // one more wave streaming a 16 KiB step at 6.0 TB/s
+  int best_ps = 256;
+  double best_t = 1e30;
   for (int parts = 1;; ++parts) {
     int ps = (max_context_len + parts - 1) / parts;
     ps = (ps + 255) / 256 * 256;
     int w = ps >= 1024 ? 4 : (ps >= 512 ? 2 : 1);
     w = w > cap_w ? cap_w : w;
-    if (ps <= 256) return 256;
-    if (ps <= 2048 * w && rows * parts * w >= slots) return ps;
+    if (ps <= 2048 * w) {
+      const int steps_per_wave = ((ps + 63) / 64 + w - 1) / w;
+      const double waves = rows * parts * w;
+      const double step_us = waves * step_us_per_wave > 1.4 ? waves * step_us_per_wave : 1.4;
+      const double t = steps_per_wave * step_us + (parts > 1 ? 7.0 + 0.002 * rows * parts : 0.0);
+      if (t < best_t * 0.999) {  // ties go to fewer partitions
+        best_t = t;
+        best_ps = ps;
+      }
+    }
+    if (ps <= 256) return best_ps;
   }
 }
 
