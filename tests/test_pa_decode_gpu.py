@@ -353,6 +353,19 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("name", ["fp8_g8", "fp8_token_g16_q4", "fp8_g10_q3"])
+@pytest.mark.parametrize("gain", [4.0, 12.0])
+def test_large_logits(cuda, name, gain):
+    """Queries scaled up until the scaled logits reach tens (sharp softmax, as trained models produce): the
+    FP8 MFMAs must see the bf16 query exactly (a power-of-two row factor makes head + residual exact), or the
+    logit error, proportional to the logit, breaks the output tolerance."""
+    wl = _make(**CASES[name])
+    wl = type(wl)(**{**wl.__dict__, "query": (wl.query.float() * gain).to(wl.query.dtype)})
+    out, res = _run(wl, cuda, partition_size=512)
+    torch.testing.assert_close(out.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+    _check_stages(wl, res, 512)
+
+
 @pytest.mark.parametrize("case", ["queue", "sorted", "plain"])
 def test_graph_capture_and_replay(cuda, case):
     """A decode plan allocates nothing and only launches kernels on the given stream, so it can be captured

@@ -76,6 +76,21 @@ __device__ __forceinline__ float sload_f32(const float* p) {
   return *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(p));
 }
 
+// Power-of-two factor that brings a row of query values with largest magnitude amax into [128, 256): a bf16
+// (8 significant bits) or FP8 value times a power of two is then EXACTLY an e4m3 head (4 significant bits)
+// plus an e4m3 residual, so the FP8 MFMAs see the query without rounding (elements more than 2^15 below the
+// row maximum lose bits to e4m3's subnormal range: an absolute error below 2^-17 of the row maximum).
+// inv receives 1 / factor.  amax == 0 (or not finite) gives 1.
+__device__ __forceinline__ float query_pow2_factor(float amax, float& inv) {
+  const int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 127;
+  if (!(amax > 0.f) || e < -100 || e > 100) {
+    inv = 1.f;
+    return 1.f;
+  }
+  inv = __uint_as_float((uint32_t)(127 - 7 + e) << 23);
+  return __uint_as_float((uint32_t)(127 + 7 - e) << 23);
+}
+
 // max / sum over the four lanes {l, l^16, l^32, l^48}: v_permlane{16,32}_swap exchange 16- and
 // 32-lane halves inside the VALU (no LDS round trip)
 __device__ __forceinline__ float quad_row_max(float x) {

@@ -341,7 +341,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       qs = a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
     rscale[nt] = scale2 * qs;
   }
-  // FP8 math: q * cq = hi + lo with hi, lo in e4m3 (|q * cq| <= 224); the logits are divided by cq again
+  // FP8 math: q * cq = hi + lo with hi, lo in e4m3 and cq a power of two (exact); the logits are divided by cq again
   i32x8 qhi[FP8MATH ? NT : 1], qlo[FP8MATH ? NT : 1];
   if constexpr (FP8MATH) {
 #pragma unroll
@@ -361,8 +361,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 #pragma unroll
       for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(f[e]));
       amax = quad_row_max(amax);
-      const float cq = amax > 0.f ? 224.f / amax : 1.f;
-      rscale[nt] *= amax > 0.f ? amax * (1.f / 224.f) : 1.f;
+      float cq_inv;
+      const float cq = query_pow2_factor(amax, cq_inv);
+      rscale[nt] *= cq_inv;
 #pragma unroll
       for (int w = 0; w < 8; ++w) {
         const float x0 = f[4 * w] * cq, x1 = f[4 * w + 1] * cq, x2 = f[4 * w + 2] * cq, x3 = f[4 * w + 3] * cq;

@@ -161,7 +161,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   if (has_alibi && row_ok) slope2 = a.alibi_slopes[h * G + (row - t_row * G)] * kLog2e;
   const int min_limit = ctx - (qb - 1);
 
-  // ---- query: q * cq = hi + lo in e4m3 (|q * cq| <= 224), the B operand of S^T = K Q^T -------------------
+  // ---- query: q * cq = hi + lo in e4m3, cq a power of two (exact), the B operand of S^T = K Q^T ---------
   float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
   if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
     k_tensor_scale = sload_f32(a.key_scale);
@@ -197,8 +197,9 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
 #pragma unroll
     for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(f[e]));
     amax = quad_row_max(amax);
-    const float cq = amax > 0.f ? 224.f / amax : 1.f;
-    rscale *= amax > 0.f ? amax * (1.f / 224.f) : 1.f;
+    float cq_inv;
+    const float cq = query_pow2_factor(amax, cq_inv);
+    rscale *= cq_inv;
 #pragma unroll
     for (int w = 0; w < 8; ++w) {
       const float x0 = f[4 * w] * cq, x1 = f[4 * w + 1] * cq, x2 = f[4 * w + 2] * cq, x3 = f[4 * w + 3] * cq;

@@ -65,10 +65,11 @@ class DecodePlan:
     """A validated call: the filled C struct plus the tensors it points to (kept alive).
     `run()` enqueues partition + reduce on a stream; it allocates nothing and can be replayed."""
 
-    def __init__(self, args: PaDecodeArgs, keep, exp_sums, max_logits, tmp_output, output):
+    def __init__(self, args: PaDecodeArgs, keep, exp_sums, max_logits, tmp_output, output, workspace=None):
         self.args = args
         self._keep = keep
         self.exp_sums, self.max_logits, self.tmp_output, self.output = exp_sums, max_logits, tmp_output, output
+        self.workspace = workspace
         self._lib = _cabi.load_library()
 
     def run(self, stream: Optional[int] = None) -> None:
@@ -315,7 +316,7 @@ def plan_decode(
     a.stride_qscale_s, a.stride_kvscale_b, a.stride_kvscale_h = stride_qs, stride_kvs_b, stride_kvs_h
     keep = (output, query, key_cache, value_cache, sequence_lengths, block_tables, query_scale, key_scale,
             value_scale, alibi_slopes, query_lens, workspace, sinks)
-    return DecodePlan(a, keep, exp_sums, max_logits, tmp_output, output)
+    return DecodePlan(a, keep, exp_sums, max_logits, tmp_output, output, workspace)
 
 
 def paged_attention_decode(
