@@ -2,12 +2,13 @@
 raw ctypes functions), against the CPU oracle on the same seeded inputs.
 
 Tolerances.  End to end the bar is atol 2e-2 / rtol 2e-2 on the bf16 output (torch.allclose rule
-|a-b| <= atol + rtol*|b|).  Stage-wise: with an FP8 cache the kernel multiplies the cache bytes on the
-FP8 MFMAs and carries the bf16 query as an FP8 head plus an FP8 residual (about 2^-8 relative per
-element, like bf16 itself), so a scaled logit differs from the f32 oracle by a few 1e-3: max_logits
-is compared at atol 4e-3 + rtol 2e-3 and exp_sums at rtol 1e-2; with a bf16 cache (bf16 MFMA, exact
-products) both are compared at 1e-4.  tmp_output carries the rounding of P and of the stored bf16
-value and is compared at 2e-2 like the output.
+|a-b| <= atol + rtol*|b|).  Stage-wise: the cache bytes and the query reach the MFMAs exactly (a bf16
+cache on the bf16 MFMAs; an FP8 cache on the FP8 MFMAs with the bf16 query carried as an FP8 head plus
+an FP8 residual under a power-of-two row factor, which is exact), so max_logits and exp_sums differ
+from the f32 oracle by accumulation order only and are compared at 1e-4 (bf16 cache) / 5e-4 (FP8 cache,
+whose scales are applied in another order).  tmp_output carries the
+rounding of P (about 2^-8 relative per element) and of the stored bf16 value and is compared at 2e-2
+like the output.
 """
 import ctypes as C
 import math
@@ -56,12 +57,14 @@ def _check_stages(wl, res, partition_size, alibi=None):
     gto = res["temporary_output"].float().cpu()
     fin = torch.isfinite(ml)
     assert torch.equal(gml[~fin], ml[~fin]), "rows with no visible key must hold max=-inf"
+    # the cache bytes and the query enter the MFMAs exactly (bf16, or FP8 with the query as an exact FP8
+    # head + residual): the logits differ from the f32 oracle by accumulation order only
     if wl.key_cache.dtype == torch.bfloat16:
         torch.testing.assert_close(gml[fin], ml[fin], atol=1e-4, rtol=1e-5)
         torch.testing.assert_close(ges, es, atol=1e-4, rtol=1e-4)
-    else:
-        torch.testing.assert_close(gml[fin], ml[fin], atol=4e-3, rtol=2e-3)
-        torch.testing.assert_close(ges, es, atol=1e-3, rtol=1e-2)
+    else:  # the scales are applied in another order (folded into the exponent): a few f32 roundings more
+        torch.testing.assert_close(gml[fin], ml[fin], atol=5e-4, rtol=5e-5)
+        torch.testing.assert_close(ges, es, atol=5e-4, rtol=1e-3)
     torch.testing.assert_close(gto, to, atol=ATOL, rtol=RTOL)
     # the reduce kernel alone, on the kernel's own partition buffers, against the closed-form merge
     merged = O.reduce_stage(gml, ges, gto, wl.context_lens, partition_size)
