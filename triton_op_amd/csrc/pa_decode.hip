@@ -146,17 +146,25 @@ int tiles_per_workgroup(int total_tiles) {
   return t < total_tiles ? t : total_tiles;
 }
 
-// Waves per workgroup: about 256 tokens (4 steps) per wave at least, and at most 4 / NT waves (the
-// merge buffer of a workgroup is NT * WAVES * 8 KiB of LDS).
+// Waves per workgroup: 128 tokens (2 steps) per wave at least, and at most 4 / NT waves (the merge buffer of a
+// workgroup is NT * WAVES * 8 KiB of LDS).  Eight waves (one partition where four waves take two) were
+// measured and lose: a wave's chain of 1.4 us steps is what a small batch waits for, and more partitions
+// shorten it where more waves per workgroup cannot go below the second kernel's cost anyway.
+int waves_for_partition_size(int partition_size, int nt) {
+  int w = partition_size >= 512 ? 4 : 2;
+  const int cap = nt == 1 ? 4 : (nt == 2 ? 2 : 1);
+  return w > cap ? cap : w;
+}
 int waves_per_workgroup(const PaDecodeArgs& a, int nt) {
   static const int forced = [] {
     const char* e = getenv("PA_DECODE_WAVES");
     return e ? atoi(e) : 0;
   }();
-  int w = a.partition_size >= 1024 ? 4 : (a.partition_size >= 512 ? 2 : 1);
-  if (forced > 0) w = forced;
-  const int cap = nt == 1 ? 4 : (nt == 2 ? 2 : 1);
-  w = w > cap ? cap : w;
+  int w = waves_for_partition_size(a.partition_size, nt);
+  if (forced > 0) {
+    const int cap = nt == 1 ? 4 : (nt == 2 ? 2 : 1);
+    w = forced > cap ? cap : forced;
+  }
   return w >= 4 ? 4 : (w >= 2 ? 2 : 1);
 }
 
@@ -288,18 +296,17 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
       if (ps <= 8192 && items * parts >= slots) return ps;
     }
   }
-  // One workgroup per 16-row query tile, up to 4 waves (at least 256 tokens each) per workgroup, no wave with
+  // One workgroup per 16-row query tile, up to 4 waves (at least 128 tokens each) per workgroup, no wave with
   // more than 2048 tokens (which keeps ragged batches balanced).  The number of partitions per sequence is the
   // one a small cost model likes best (times in microseconds on this GPU):
-  //   a wave's 64-token step takes the longer of 1.4 us (one wave alone: a 16 KiB step per HBM round trip) and
-  //   its share of the HBM stream when `waves` of them run at once, 16 KiB * waves / 6.0 TB/s (more waves than
-  //   the GPU holds simply queue: the same formula);
+  //   a wave costs 1.3 us to set up, and each of its 64-token steps the longer of 1.4 us (one wave alone: a
+  //   16 KiB step per HBM round trip) and its share of the HBM stream when `waves` of them run at once,
+  //   16 KiB * waves / 6.0 TB/s (more waves than the GPU holds simply queue: the same formula);
   //   splitting a sequence costs the second kernel (7 us) and its partials (written, read back: 2 ns per
   //   16-row tile and partition).
   // Few rows and long contexts want many partitions; 256 or more rows want one, even if that leaves a quarter
   // of the wave slots empty (measured at 48 sequences x 8 kv heads x 4096 tokens: 78 us against 87 us for two).
   const int nt = tiles_per_workgroup(total_tiles);
-  const int cap_w = nt <= 1 ? 4 : 2;
   const double rows = (double)num_seqs * num_kv_heads * ((total_tiles + nt - 1) / nt);
   const double step_us_per_wave = 16384.0 / 6.0e6;  // one more wave streaming a 16 KiB step at 6.0 TB/s
   int best_ps = 256;
@@ -307,13 +314,12 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   for (int parts = 1;; ++parts) {
     int ps = (max_context_len + parts - 1) / parts;
     ps = (ps + 255) / 256 * 256;
-    int w = ps >= 1024 ? 4 : (ps >= 512 ? 2 : 1);
-    w = w > cap_w ? cap_w : w;
+    const int w = waves_for_partition_size(ps, nt);
     if (ps <= 2048 * w) {
       const int steps_per_wave = ((ps + 63) / 64 + w - 1) / w;
       const double waves = rows * parts * w;
       const double step_us = waves * step_us_per_wave > 1.4 ? waves * step_us_per_wave : 1.4;
-      const double t = steps_per_wave * step_us + (parts > 1 ? 7.0 + 0.002 * rows * parts : 0.0);
+      const double t = 1.3 + steps_per_wave * step_us + (parts > 1 ? 7.0 + 0.002 * rows * parts : 0.0);
       if (t < best_t * 0.999) {  // ties go to fewer partitions
         best_t = t;
         best_ps = ps;
