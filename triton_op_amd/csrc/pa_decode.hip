@@ -133,38 +133,21 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
 }
 
 
-// 16-row query tiles per workgroup.  More than 16 query rows per kv head (large GQA groups, MTP) are split
-// over workgroups of one tile each by default: they re-read the same pages at the same time from the
-// same L2, run the 2-waves-per-SIMD variant, and tiles that hold only padding rows cost nothing.
-// PA_DECODE_TILES=2 keeps two tiles in one workgroup (one pass over the pages, 1 wave per SIMD).
-int tiles_per_workgroup(int total_tiles) {
-  static const int forced = [] {
-    const char* e = getenv("PA_DECODE_TILES");
-    return e ? atoi(e) : 0;
-  }();
-  const int t = forced == 2 ? 2 : 1;
-  return t < total_tiles ? t : total_tiles;
-}
-
-// Waves per workgroup: 128 tokens (2 steps) per wave at least, and at most 4 / NT waves (the merge buffer of a
-// workgroup is NT * WAVES * 8 KiB of LDS).  Eight waves (one partition where four waves take two) were
+// pa_partition_kernel is instantiated with one 16-row query tile per workgroup (NT = 1): a bf16 cache with
+// more than 16 query rows per kv head gets one workgroup per tile (they read the same pages at the same time
+// from the same L2, and tiles that hold only padding rows cost nothing); an FP8 cache goes to
+// pa_partition_shared_kernel.
+// Waves per workgroup: 128 tokens (2 steps) per wave at least, and at most 4 waves (the merge buffer of a
+// workgroup is WAVES * 8 KiB of LDS).  Eight waves (one partition where four waves take two) were
 // measured and lose: a wave's chain of 1.4 us steps is what a small batch waits for, and more partitions
 // shorten it where more waves per workgroup cannot go below the second kernel's cost anyway.
-int waves_for_partition_size(int partition_size, int nt) {
-  int w = partition_size >= 512 ? 4 : 2;
-  const int cap = nt == 1 ? 4 : (nt == 2 ? 2 : 1);
-  return w > cap ? cap : w;
-}
-int waves_per_workgroup(const PaDecodeArgs& a, int nt) {
+int waves_for_partition_size(int partition_size) { return partition_size >= 512 ? 4 : 2; }
+int waves_per_workgroup(const PaDecodeArgs& a) {
   static const int forced = [] {
     const char* e = getenv("PA_DECODE_WAVES");
     return e ? atoi(e) : 0;
   }();
-  int w = waves_for_partition_size(a.partition_size, nt);
-  if (forced > 0) {
-    const int cap = nt == 1 ? 4 : (nt == 2 ? 2 : 1);
-    w = forced > cap ? cap : forced;
-  }
+  const int w = forced > 0 ? forced : waves_for_partition_size(a.partition_size);
   return w >= 4 ? 4 : (w >= 2 ? 2 : 1);
 }
 
@@ -205,18 +188,11 @@ int launch_partition_shared(const PaDecodeArgs& a, hipStream_t stream) {
 }
 
 template <int KVT, bool PT, bool BS16>
-int launch_partition_nt(const PaDecodeArgs& a, int nt, hipStream_t stream) {
-  const int w = waves_per_workgroup(a, nt);
-  switch (nt) {
-    case 1:
-      if (w == 4) return launch_partition_w<1, KVT, PT, BS16, 4>(a, stream);
-      if (w == 2) return launch_partition_w<1, KVT, PT, BS16, 2>(a, stream);
-      return launch_partition_w<1, KVT, PT, BS16, 1>(a, stream);
-    case 2:
-      if (w == 2) return launch_partition_w<2, KVT, PT, BS16, 2>(a, stream);
-      return launch_partition_w<2, KVT, PT, BS16, 1>(a, stream);
-  }
-  return PA_ERR_UNSUPPORTED;
+int launch_partition_tile(const PaDecodeArgs& a, hipStream_t stream) {
+  const int w = waves_per_workgroup(a);
+  if (w == 4) return launch_partition_w<1, KVT, PT, BS16, 4>(a, stream);
+  if (w == 2) return launch_partition_w<1, KVT, PT, BS16, 2>(a, stream);
+  return launch_partition_w<1, KVT, PT, BS16, 1>(a, stream);
 }
 
 int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
@@ -306,15 +282,14 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   //   16-row tile and partition).
   // Few rows and long contexts want many partitions; 256 or more rows want one, even if that leaves a quarter
   // of the wave slots empty (measured at 48 sequences x 8 kv heads x 4096 tokens: 78 us against 87 us for two).
-  const int nt = tiles_per_workgroup(total_tiles);
-  const double rows = (double)num_seqs * num_kv_heads * ((total_tiles + nt - 1) / nt);
+  const double rows = (double)num_seqs * num_kv_heads * total_tiles;
   const double step_us_per_wave = 16384.0 / 6.0e6;  // one more wave streaming a 16 KiB step at 6.0 TB/s
   int best_ps = 256;
   double best_t = 1e30;
   for (int parts = 1;; ++parts) {
     int ps = (max_context_len + parts - 1) / parts;
     ps = (ps + 255) / 256 * 256;
-    const int w = waves_for_partition_size(ps, nt);
+    const int w = waves_for_partition_size(ps);
     if (ps <= 2048 * w) {
       const int steps_per_wave = ((ps + 63) / 64 + w - 1) / w;
       const double waves = rows * parts * w;
@@ -358,7 +333,6 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
     return PA_ERR_BAD_SHAPE;
 
   const int Ge = a->q_len * a->group_size;
-  const int nt = tiles_per_workgroup((Ge + 15) / 16);
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   const bool pt = a->kv_quant_mode == PA_QUANT_PER_TOKEN;
   if (a->kv_dtype == PA_DTYPE_FP8_E4M3FN) {
@@ -370,13 +344,13 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
       return pt ? launch_partition_shared<true, false>(*a, stream) : launch_partition_shared<false, false>(*a, stream);
     }
     if (bs16)
-      return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, true>(*a, nt, stream)
-                : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, true>(*a, nt, stream);
-    return pt ? launch_partition_nt<PA_DTYPE_FP8_E4M3FN, true, false>(*a, nt, stream)
-              : launch_partition_nt<PA_DTYPE_FP8_E4M3FN, false, false>(*a, nt, stream);
+      return pt ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, true>(*a, stream)
+                : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, true>(*a, stream);
+    return pt ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, false>(*a, stream)
+              : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, false>(*a, stream);
   }
   if (pt) return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
-  return launch_partition_nt<PA_DTYPE_BF16, false, false>(*a, nt, stream);
+  return launch_partition_tile<PA_DTYPE_BF16, false, false>(*a, stream);
 }
 
 int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) { return launch_reduce(a, hip_stream, false); }
