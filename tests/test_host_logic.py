@@ -193,3 +193,35 @@ def test_graft_entry_points_exist():
     import __graft_entry__ as g
 
     assert callable(g.build) and callable(g.smoke)
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """include/pa_decode.h is the contract of a foreign-function binding: it must compile as C99 on its own, and a
+    C program that uses it must link against the library and see the same struct size."""
+    import os
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "use_abi.c"
+    src.write_text(
+        '#include <stdio.h>\n#include "pa_decode.h"\n'
+        "int main(void) {\n"
+        "  PaDecodeArgs a = {0};\n"
+        "  a.struct_size = sizeof a;\n"
+        "  if (pa_decode_abi_version() != PA_DECODE_ABI_VERSION) return 2;\n"
+        "  if (pa_decode_args_size() != sizeof(PaDecodeArgs)) return 3;\n"
+        "  if (pa_decode(&a, 0) != PA_ERR_NULL_POINTER) return 4;  /* buffers are NULL: rejected before any launch */\n"
+        '  printf("%s\\n", pa_decode_error_string(PA_ERR_BAD_SHAPE));\n'
+        "  return 0;\n}\n")
+    exe = tmp_path / "use_abi"
+    libdir = os.path.join(root, "triton_op_amd")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(root, "include"), str(src),
+                    "-L", libdir, "-lpa_decode", "-Wl,-rpath," + libdir, "-o", str(exe)], check=True,
+                   capture_output=True, text=True)
+    res = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert res.returncode == 0, (res.returncode, res.stdout, res.stderr)
+    assert "stride" in res.stdout or "size" in res.stdout
