@@ -59,16 +59,18 @@ int device_num_cus() {
   return n;
 }
 
-// The queued launch is used when the caller gave a workspace and per-sequence query lengths (row tiles of
-// padding rows are then common): a resident grid pulls live items from a counter.  Without query lengths
-// the only workgroups with nothing to do are partitions past a sequence's end, which the plain launch
-// orders last; there the queue's bookkeeping costs more than it saves (measured: +10 % on a uniform batch).
+// The queued launch is used when the caller gave a workspace and per-sequence query lengths and a kv head has
+// more than one 16-row query tile (tiles of padding rows only are then common): a resident grid pulls live
+// items from a counter.  Otherwise the only workgroups with nothing to do are partitions past a sequence's end,
+// which the plain launch orders last; there the queue's bookkeeping costs more than it saves (measured: +10 %
+// on a uniform batch).
 bool use_queue(const PaDecodeArgs& a) {
   static const bool off = [] {
     const char* e = getenv("PA_DECODE_QUEUE");
     return e && e[0] == '0';
   }();
-  return !off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr;
+  return !off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr &&
+         a.q_len * a.group_size > 16;
 }
 
 // Bytes of workspace the sorted dispatch needs: the header and one (sequence, partition) pair per possible item.
