@@ -282,8 +282,8 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   // One workgroup per 16-row query tile, up to 4 waves (at least 128 tokens each) per workgroup, no wave with
   // more than 2048 tokens (which keeps ragged batches balanced).  The number of partitions per sequence is the
   // one a small cost model likes best (times in microseconds on this GPU):
-  //   a wave costs 1.3 us to set up, and each of its 64-token steps the longer of 1.4 us (one wave alone: a
-  //   16 KiB step per HBM round trip) and its share of the HBM stream when `waves` of them run at once,
+  //   a wave costs 1.3 us to set up, and each of its 64-token steps the longer of 1.4 us (one wave alone: the
+  //   step's own chain of loads, MFMAs and softmax) and its share of the HBM stream when `waves` of them run at once,
   //   16 KiB * waves / 6.0 TB/s (more waves than the GPU holds simply queue: the same formula);
   //   splitting a sequence costs the second kernel (7 us) and its partials (written, read back: 2 ns per
   //   16-row tile and partition).
