@@ -356,6 +356,36 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("case", ["one_partition", "partitions", "shared", "sorted", "queue"])
+def test_empty_sequences_get_zero_rows(cuda, case):
+    """A sequence with context length 0 has nothing to attend to: its output rows are zero in every launch mode
+    (also when no reduce kernel runs), and its neighbours are unaffected."""
+    import triton_op_amd as T
+
+    kw, ps = dict(
+        one_partition=(dict(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(100, 0, 200, 0)), 256),
+        partitions=(dict(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(700, 0, 200, 0)), 256),
+        shared=(dict(batch=4, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(100, 0, 200, 0), q_len=3), 256),
+        sorted=(dict(batch=96, num_q_heads=16, num_kv_heads=8,
+                     context_lens=torch.cat([_ctx(0, 1500, 0), torch.randint(1, 2600, (93,),
+                                            generator=torch.Generator().manual_seed(5), dtype=torch.int32)])), 256),
+        queue=(dict(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 0, 200, 0), q_len=4,
+                    q_lens=_ctx(4, 2, 1, 4), kv_dtype="bf16", scale_mode="none"), 512),
+    )[case]
+    # the generator wants at least one page per sequence: build with length 1, then declare the sequences empty
+    empty = kw["context_lens"] == 0
+    wl = _make(**{**kw, "context_lens": torch.clamp(kw["context_lens"], min=kw.get("q_len", 1))})
+    ctx = wl.context_lens.clone()
+    ctx[empty] = 0
+    wl = type(wl)(**{**wl.__dict__, "context_lens": ctx})
+    out, _ = _run(wl, cuda, partition_size=ps)
+    assert not torch.isnan(out.float()).any()
+    assert bool((out[empty] == 0).all())
+    live = [i for i in range(len(ctx)) if not bool(empty[i])]
+    ref = _oracle(wl, seq_ids=live)
+    torch.testing.assert_close(out[live].float(), ref[live].float(), atol=ATOL, rtol=RTOL)
+
+
 @pytest.mark.parametrize("name", ["fp8_g8", "fp8_token_g16_q4", "fp8_g10_q3"])
 @pytest.mark.parametrize("gain", [4.0, 12.0])
 def test_large_logits(cuda, name, gain):

@@ -166,6 +166,18 @@ __device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)
   __builtin_amdgcn_wave_barrier();
 }
 
+// A sequence with no tokens at all (context length <= 0): nobody streams anything, and when the call has a
+// single partition per sequence no second kernel runs either, so the workgroups of partition 0 zero the
+// sequence's output rows [row_begin, row_end) of kv head h themselves.  Called by a whole workgroup.
+__device__ __forceinline__ void zero_output_rows(const PaDecodeArgs& a, int b, int h, int row_begin, int row_end) {
+  if (a.output == nullptr) return;
+  const int Ge = a.q_len * a.group_size;
+  char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+  const int li = threadIdx.x & 15;
+  for (int r = row_begin + (int)(threadIdx.x >> 4); r < row_end; r += (int)(blockDim.x >> 4))
+    *reinterpret_cast<u32x4*>(outp + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
+}
+
 // Global memory -> LDS without passing through registers: lane i's 16 (4) bytes land at lds_offset + 16 (4) * i.
 // The loads count in vmcnt like any other vector load, but the compiler does not see them: whoever reads
 // the LDS bytes waits with dma_wait<N>() (at most N vector memory operations still outstanding) first.

@@ -97,7 +97,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         const int bb = b0 + lane;
         const int c = bb < a.num_seqs ? a.context_lens[bb] : 0;
         int np = (c + a.partition_size - 1) / a.partition_size;
-        np = np < 0 ? 0 : (np > P ? P : np);
+        np = np <= 0 ? 1 : (np > P ? P : np);  // an empty sequence keeps one item: its workgroups zero its output rows
         const int ql = bb < a.num_seqs ? (a.q_lens ? a.q_lens[bb] : a.q_len) : 0;
         int tiles = (ql * a.group_size + 16 * NT - 1) / (16 * NT);
         tiles = tiles > RT ? RT : tiles;
@@ -166,7 +166,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;
-  if (wg_start >= ctx) break;
+  if (wg_start >= ctx) {
+    if (ctx <= 0 && part == 0) {
+      if constexpr (QUEUE) {  // only tiles with real query rows are items: the first one zeroes the whole group
+        if (rt == 0) zero_output_rows(a, b, h, 0, Ge);
+      } else {
+        zero_output_rows(a, b, h, row0, row0 + 16 * NT < Ge ? row0 + 16 * NT : Ge);
+      }
+    }
+    break;
+  }
   const int wg_end = min(wg_start + a.partition_size, ctx);
   // The waves take the partition's 64-token steps round robin (wave w: steps w, w + WAVES, ...), so at any
   // time the workgroup reads WAVES * 64 consecutive tokens: with large blocks that is whole 128-byte lines of

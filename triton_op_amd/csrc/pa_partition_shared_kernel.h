@@ -61,7 +61,10 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
 
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;
-  if (wg_start >= ctx) return;
+  if (wg_start >= ctx) {
+    if (ctx <= 0 && part == 0) zero_output_rows(a, b, h, 0, Ge);
+    return;
+  }
   const int wg_end = min(wg_start + a.partition_size, ctx);
   const int n_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
   const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;

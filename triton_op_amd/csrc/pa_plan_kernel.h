@@ -40,6 +40,7 @@ __global__ __launch_bounds__(1024) void pa_plan_kernel(const PaDecodeArgs a) {
       f = f > P ? P : f;
       nfull[i] = f;
       tail[i] = np > f ? c - f * ps : 0;
+      if (c == 0) tail[i] = 1;  // an empty sequence: one (shortest) item, whose workgroups zero its output rows
       mine += f;
     }
   }
