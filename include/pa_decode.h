@@ -60,7 +60,8 @@ enum {
  *   key_cache     [num_blocks, Hkv, D/x, bs, x]
  *   value_cache   [num_blocks, Hkv, D, bs]           (v_transposed = 0)
  *                 [num_blocks, Hkv, bs/x, D, x]      (v_transposed = 1)
- *   context_lens  int32 [B]   tokens in the cache for each sequence, the q new ones included
+ *   context_lens  int32 [B]   tokens in the cache for each sequence, the q new ones included (0: the
+ *                 sequence's output rows are written as zero)
  *   block_tables  int32 [B, >= ceil(ctx/bs)]
  *   q_lens        int32 [B] or NULL: per-sequence number of new tokens (1..q); rows t >= q_lens[b]
  *                 are padding and their output rows are written as zero
