@@ -67,6 +67,11 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __ui
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+// The same for bytes that are read once and never again (the K/V cache stream): a non-temporal load.  A plain
+// read-only stream reaches 6.0-6.3 TB/s on this GPU, a non-temporal one 6.7-7.0 TB/s (measured on 4 GiB).
+__device__ __forceinline__ u32x4 load16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
 
 // wave-uniform 32-bit load through the scalar (constant) path: no VGPR, no vmcnt slot
 __device__ __forceinline__ int sload_i32(const int* p) {
@@ -179,15 +184,18 @@ __device__ __forceinline__ void zero_output_rows(const PaDecodeArgs& a, int b, i
 }
 
 // Global memory -> LDS without passing through registers: lane i's 16 (4) bytes land at lds_offset + 16 (4) * i.
+// They are non-temporal (the cache is streamed once).
 // The loads count in vmcnt like any other vector load, but the compiler does not see them: whoever reads
 // the LDS bytes waits with dma_wait<N>() (at most N vector memory operations still outstanding) first.
 __device__ __forceinline__ void dma_load16(const void* gptr, uint32_t lds_offset) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_offset) : "memory");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory");
 }
 __device__ __forceinline__ void dma_load4(const void* gptr, uint32_t lds_offset) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(lds_offset) : "memory");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory");
 }
-// the same with the address split into a wave-uniform base and a 32-bit per-lane byte offset
+// the same with the address split into a wave-uniform base and a 32-bit per-lane byte offset; STREAM = false
+// for bytes whose 128-byte lines other loads will touch again soon (those must stay in L2)
+template <bool STREAM = true>
 __device__ __forceinline__ void dma_load16(const void* base, uint32_t lane_offset, uint32_t lds_offset) {
   // the base is wave-uniform by construction; readfirstlane makes the compiler keep it in scalar registers
   const uint64_t b = reinterpret_cast<uint64_t>(base);
@@ -196,9 +204,14 @@ __device__ __forceinline__ void dma_load16(const void* base, uint32_t lane_offse
   const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
   const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
   const uint64_t sb = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(sb),
-               "s"(lds_offset)
-               : "memory");
+  if constexpr (STREAM)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" ::"v"(lane_offset), "s"(sb),
+                 "s"(lds_offset)
+                 : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(sb),
+                 "s"(lds_offset)
+                 : "memory");
 }
 template <int N>
 __device__ __forceinline__ void dma_wait() {

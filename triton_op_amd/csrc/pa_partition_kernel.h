@@ -226,6 +226,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // (with block size 16 the plain and the transposed FP8 layouts are the same bytes; for bf16 they
   // differ, so the constant-stride form is used for the plain layout only)
   const bool vt = a.v_transposed;
+  const bool v_whole_lines = KVT == PA_DTYPE_FP8_E4M3FN && (a.v_transposed || a.block_size <= 64);
   const uint32_t v_row_bytes = BS16 ? 16u * esz : (vt ? 16u : (uint32_t)(a.stride_v_2 * esz));
   const uint32_t v_half_bytes = BS16 ? 16u : (vt ? (uint32_t)(a.stride_v_2 * esz) : 16u);
   const int64_t v_tile_bytes = BS16 ? 16 * esz : (vt ? a.stride_v_2 * esz * esz : 16 * esz);
@@ -258,7 +259,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     for (int j = 0; j < 4; ++j) {
       const char* tb = kbase + (int64_t)pg.p[j] * k_block_bytes + (int64_t)pg.off[j] * 16;
 #pragma unroll
-      for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16(tb + k_lane_off[ld]);
+      for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16_stream(tb + k_lane_off[ld]);
       if constexpr (PER_TOKEN) {
         const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + pg.off[j] + 4 * kg;
         sd.ks[j] = *reinterpret_cast<const f32x4*>(ksbase + so);
@@ -270,10 +271,21 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     const int page = kg == 0 ? pg.p[0] : (kg == 1 ? pg.p[1] : (kg == 2 ? pg.p[2] : pg.p[3]));
     const int off = kg == 0 ? pg.off[0] : (kg == 1 ? pg.off[1] : (kg == 2 ? pg.off[2] : pg.off[3]));
     const char* tb = vbase + (int64_t)page * v_block_bytes + (int64_t)(off >> 4) * v_tile_bytes;
+    // Non-temporal where one load covers whole 128-byte lines.  With plain V and pages of more than 64 tokens
+    // a 64-token step takes half a line of every head dim's row and the next step the other half: those lines
+    // must stay in L2 in between (streaming them costs 13 % on 1024-token pages).
+    if (BS16 || v_whole_lines) {
 #pragma unroll
-    for (int db = 0; db < 8; ++db) {
+      for (int db = 0; db < 8; ++db) {
 #pragma unroll
-      for (int hf = 0; hf < SD::NVL; ++hf) sd.v[db][hf] = load16(tb + v_lane_off[db] + hf * v_half_bytes);
+        for (int hf = 0; hf < SD::NVL; ++hf) sd.v[db][hf] = load16_stream(tb + v_lane_off[db] + hf * v_half_bytes);
+      }
+    } else {
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+#pragma unroll
+        for (int hf = 0; hf < SD::NVL; ++hf) sd.v[db][hf] = load16(tb + v_lane_off[db] + hf * v_half_bytes);
+      }
     }
     if constexpr (PER_TOKEN) {
 #pragma unroll

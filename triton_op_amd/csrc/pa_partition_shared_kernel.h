@@ -90,6 +90,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
 #pragma unroll
   for (int ld = 0; ld < 2; ++ld) k_lane_off[ld] = (uint32_t)(kg * k_chunk_bytes + li * 16) + 4 * ld * k_chunk_bytes;
   const bool vt = a.v_transposed;
+  const bool v_whole_lines = a.v_transposed || a.block_size <= 64;
   const uint32_t v_row_bytes = BS16 ? 16u : (vt ? 16u : (uint32_t)a.stride_v_2);
   const int64_t v_tile_bytes = BS16 ? 16 : (vt ? a.stride_v_2 : 16);
   uint32_t v_lane_off[2];  // V loads: lane = head dim (0..63, 64..127) of one tile
@@ -126,8 +127,15 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     dma_load16(kt, k_lane_off[1], kdst + 1024u);
     const char* vt_ = vbase + (int64_t)page * v_block_bytes + (int64_t)(off >> 4) * v_tile_bytes;
     const uint32_t vdst = st + (uint32_t)offsetof(StepLds, v) + (uint32_t)wave * 2048u;
-    dma_load16(vt_, v_lane_off[0], vdst);   // head dims 0..63 (lane = dim)
-    dma_load16(vt_, v_lane_off[1], vdst + 1024u);  // head dims 64..127
+    // non-temporal where a load covers whole 128-byte lines; plain V in pages of more than 64 tokens gives a
+    // step half a line of every head dim's row, and the other half must still be in L2 for the next step
+    if (BS16 || v_whole_lines) {
+      dma_load16<true>(vt_, v_lane_off[0], vdst);            // head dims 0..63 (lane = dim)
+      dma_load16<true>(vt_, v_lane_off[1], vdst + 1024u);    // head dims 64..127
+    } else {
+      dma_load16<false>(vt_, v_lane_off[0], vdst);
+      dma_load16<false>(vt_, v_lane_off[1], vdst + 1024u);
+    }
     if constexpr (PER_TOKEN) {
       // lanes 0-15: the K scales of the tile's 16 tokens, lanes 16-31: the V scales
       if (lane < 32)
