@@ -80,7 +80,11 @@ def test_partition_size_choices():
     assert f(4, 8, 32, 131072, 16, 256) == 5632    # few long sequences, 2 row tiles: 24 partitions fill the GPU
     assert f(4, 1, 8, 1024, 16, 256) == 1024       # c1: tiny; one partition, no second kernel
     assert f(48, 8, 8, 4096, 16, 256) == 4096      # three quarters of the wave slots filled: still one partition
-    assert f(4, 8, 8, 4096, 16, 256) == 1024       # 32 rows only: four partitions each
+    assert f(4, 8, 8, 4096, 16, 256) == 512        # 32 rows only: eight partitions each
+    assert f(8, 8, 8, 4096, 16, 256) == 512        # measured 18.6 us against 20.2 (1024) and 27.6 (4096)
+    assert f(16, 8, 8, 4096, 16, 256) == 1024      # measured 29.2 us against 30.8 (512) and 30.6 (4096)
+    assert f(24, 8, 8, 4096, 16, 256) == 4096      # measured 36.4 us against 41.5 (2048)
+    assert f(1, 8, 8, 4096, 16, 256) == 512
     for args in [(1, 1, 1, 1, 16, 256), (3, 5, 7, 100000, 64, 304), (1000, 8, 16, 300, 16, 64)]:
         ps = f(*args)
         assert ps >= 256 and ps % 256 == 0

@@ -282,15 +282,18 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
   // One workgroup per 16-row query tile, up to 4 waves (at least 128 tokens each) per workgroup, no wave with
   // more than 2048 tokens (which keeps ragged batches balanced).  The number of partitions per sequence is the
   // one a small cost model likes best (times in microseconds on this GPU):
-  //   a wave costs 1.3 us to set up, and each of its 64-token steps the longer of 1.4 us (one wave alone: the
-  //   step's own chain of loads, MFMAs and softmax) and its share of the HBM stream when `waves` of them run at once,
-  //   16 KiB * waves / 6.0 TB/s (more waves than the GPU holds simply queue: the same formula);
+  //   a wave costs 1.3 us to set up; each of its 64-token steps costs the root sum of squares of 1.4 us (one
+  //   wave alone: the step's own chain of loads, MFMAs and softmax) and its share of the HBM stream when
+  //   `waves` of them run at once, 16 KiB * waves / 6.5 TB/s; the GPU holds 8 waves per CU, more run in rounds;
   //   splitting a sequence costs the second kernel (7 us) and its partials (written, read back: 2 ns per
   //   16-row tile and partition).
   // Few rows and long contexts want many partitions; 256 or more rows want one, even if that leaves a quarter
-  // of the wave slots empty (measured at 48 sequences x 8 kv heads x 4096 tokens: 78 us against 87 us for two).
+  // of the wave slots empty (measured at 48 sequences x 8 kv heads x 4096 tokens: 71 us against 78 us for two).
+  // Measured against sweeps over 256..4096 at 1..64 sequences of 4096 tokens: the choice is the best or within
+  // 2 % of it.
   const double rows = (double)num_seqs * num_kv_heads * total_tiles;
-  const double step_us_per_wave = 16384.0 / 6.0e6;  // one more wave streaming a 16 KiB step at 6.0 TB/s
+  const double step_us_per_wave = 16384.0 / 6.5e6;  // one more wave streaming a 16 KiB step at 6.5 TB/s
+  const double wave_slots = 8.0 * num_cus;
   int best_ps = 256;
   double best_t = 1e30;
   for (int parts = 1;; ++parts) {
@@ -300,8 +303,11 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
     if (ps <= 2048 * w) {
       const int steps_per_wave = ((ps + 63) / 64 + w - 1) / w;
       const double waves = rows * parts * w;
-      const double step_us = waves * step_us_per_wave > 1.4 ? waves * step_us_per_wave : 1.4;
-      const double t = 1.3 + steps_per_wave * step_us + (parts > 1 ? 7.0 + 0.002 * rows * parts : 0.0);
+      const double at_once = waves < wave_slots ? waves : wave_slots;
+      const double rounds = waves / at_once;
+      const double share = at_once * step_us_per_wave;
+      const double step_us = __builtin_sqrt(1.4 * 1.4 + share * share);
+      const double t = rounds * (1.3 + steps_per_wave * step_us) + (parts > 1 ? 7.0 + 0.002 * rows * parts : 0.0);
       if (t < best_t * 0.999) {  // ties go to fewer partitions
         best_t = t;
         best_ps = ps;
