@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # the counter reads for a plain copy of known size (profiles/pa_partition_kernel_c2_hbm_traffic.md,
 # profiles/pa_partition_shared_kernel_c5_hbm_traffic.md); keyed by (workload, partition size) because the
 # partial-output traffic depends on the partitioning
-HBM_TRAFFIC_BYTES = {("c2_fp8_b64_ctx4k", 4096): 541_400_000, ("c5_ragged_mix", 7424): 2_050_800_000}
+HBM_TRAFFIC_BYTES = {("c2_fp8_b64_ctx4k", 4096): 541_400_000, ("c5_ragged_mix", 7424): 2_050_400_000}
 
 
 def _partition_kernel_name(wl):
