@@ -2,6 +2,7 @@
 """Benchmark of the paged-attention decode hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--partition-size N]
+    python bench.py --workload kv_write | kv_quantize      (the KV-cache write kernels, the step before the path)
 
 A step is one call of the op (partition kernel + reduce kernel on one stream) on one batch of
 synthetic input that is already resident in HBM.  Consecutive steps use different KV pools so the
@@ -74,6 +75,102 @@ def _cpu_baseline(wl_cpu_sample, n_seq_sample, target_seconds=20.0):
 _FULL_BATCH = [0]
 
 
+def _bench_kv_cache(a) -> int:
+    """The step before the decode path: `kv_write` appends 64 prompts of 4096 tokens (8 kv heads, head 128, bf16
+    rows) to an FP8 paged cache with per-token scales in one call; `kv_quantize` converts the c2 cache pool
+    (20480 pages of 16 tokens) from bf16 to FP8 with per-token scales.  Bytes counted: rows or cache read once,
+    cache and scales written once."""
+    import torch
+
+    import triton_op_amd as T
+    from triton_op_amd import _cabi
+    from triton_op_amd import kv_layout as L
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    _cabi.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    h, d, bs = 8, 128, 16
+    gen = torch.Generator(device=dev).manual_seed(7)
+    if a.workload == "kv_write":
+        ntok = 64 * 4096
+        nblk = ntok // bs
+        key = torch.randn(ntok, h, d, device=dev, generator=gen).to(torch.bfloat16)
+        value = torch.randn(ntok, h, d, device=dev, generator=gen).to(torch.bfloat16)
+        perm = torch.randperm(nblk, device=dev, generator=gen)
+        slots = (perm.repeat_interleave(bs) * bs + torch.arange(ntok, device=dev) % bs).to(torch.int64)
+        kc = torch.zeros(nblk, h, d // 16, bs, 16, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        vc = torch.zeros(nblk, h, d, bs, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        ks = torch.zeros(nblk, h, bs, 1, device=dev)
+        vs = torch.zeros(nblk, h, bs, 1, device=dev)
+        nbytes = ntok * h * (2 * d * 2 + 2 * d + 8)
+        kernel, name = "kv_cache_write_tile_kernel", "kv_write_64x4096_fp8_token_scales"
+
+        def step():
+            T.kv_cache_write(key, value, kc, vc, slots, ks, vs)
+
+        def cpu_sample():
+            n = 4096
+            k16 = L.tokens_to_key_cache(key[:n].cpu().view(n // bs, bs, h, d))
+            v16 = L.tokens_to_value_cache(value[:n].cpu().view(n // bs, bs, h, d))
+            t0 = time.perf_counter()
+            L.quantize_kv_cache_per_token(k16, v16)
+            return n * h * (2 * d * 2 + 2 * d + 8), time.perf_counter() - t0, f"{n} tokens"
+    else:
+        nblk = 20480
+        kc16 = torch.randn(nblk, h, d // 8, bs, 8, device=dev, generator=gen).to(torch.bfloat16)
+        vc16 = torch.randn(nblk, h, d, bs, device=dev, generator=gen).to(torch.bfloat16)
+        nbytes = nblk * bs * h * (2 * d * 2 + 2 * d + 8)
+        kernel, name = "quantize_kv_cache_tile_kernel", "kv_quantize_c2_pool"
+
+        def step():
+            T.quantize_kv_cache_symmetric(kc16, vc16, torch.float8_e4m3fn)
+
+        def cpu_sample():
+            n = 256
+            k16, v16 = kc16[:n].cpu(), vc16[:n].cpu()
+            t0 = time.perf_counter()
+            L.quantize_kv_cache_per_token(k16, v16)
+            return n * bs * h * (2 * d * 2 + 2 * d + 8), time.perf_counter() - t0, f"{n} pages"
+    stream = torch.cuda.current_stream(dev)
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    t0 = time.perf_counter()
+    for e0, e1 in evs:
+        e0.record(stream)
+        step()
+        e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
+    us_median = us[len(us) // 2]
+    achieved = nbytes / (us_median * 1e-6) / 1e9
+    result = {
+        "metric": "KV-cache write GB/s (rows read + FP8 cache and scales written)", "value": round(achieved, 1),
+        "unit": "GB/s", "us_per_call": round(us_median, 2), "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 in, fp8_e4m3fn + f32 scales out", "data": "synthetic",
+        "config": {"workload": name, "kv_heads": h, "head_size": d, "block_size": bs, "bytes_per_call": nbytes},
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+    }
+    if not a.no_cpu_baseline:
+        cpu_sample()  # warm-up
+        tot_b, tot_dt, reps = 0, 0.0, 0
+        while tot_dt < 10.0:  # a bounded sample, about 10 s of host work
+            b, dt, what = cpu_sample()
+            tot_b, tot_dt, reps = tot_b + b, tot_dt + dt, reps + 1
+        result["cpu_baseline"] = {"value": round(tot_b / tot_dt / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
+                                  "kind": "port",
+                                  "sample": f"the torch formulas of kv_layout, {reps} passes over {what}, {tot_dt:.1f} s"}
+    print(json.dumps(result, ensure_ascii=False))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -89,6 +186,9 @@ def main() -> int:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op shards by kv head or "
               "by sequence with no exchange); run with --gpus 1", file=sys.stderr)
         return 2
+
+    if a.workload in ("kv_write", "kv_quantize"):
+        return _bench_kv_cache(a)
 
     import torch
 

@@ -92,3 +92,109 @@ def test_cache_write_then_decode(cuda, mode):
     torch.cuda.synchronize()
     ref = O.paged_attention_decode_oracle(q, kref, vref, ctx, bt, d ** -0.5, 1, ksr, vsr)
     torch.testing.assert_close(out.float().cpu(), ref.float(), atol=2e-2, rtol=2e-2)
+
+
+def _prefill_like_slots(bs, gen):
+    """A token stream that mixes what a serving engine sends: whole prompts of odd lengths (runs that start a
+    page), continuations of earlier chunks (runs that start in the middle of a page, also in the middle of a
+    16-slot segment), a stretch of single scattered tokens (decode rows), and padding tokens (slot -1)."""
+    runs = []  # (first slot, length) or (-1, length) for padding
+    page = 0
+
+    def new_pages(n):
+        nonlocal page
+        first = page
+        page += n
+        return first
+
+    for length in (1, 15, 16, 17, 100, 333, 1024, 31, 640):  # prompts from the start of a page
+        p = new_pages((length + bs - 1) // bs)
+        runs.append((p * bs, length))
+    for start, length in ((5, 40), (bs - 1, 18), (16 % bs, 200), (9, 3)):  # continuations at an offset
+        p = new_pages((start + length + bs - 1) // bs)
+        runs.append((p * bs + start, length))
+    runs.append((-1, 3))
+    for _ in range(70):  # scattered single tokens, every one in a page of its own
+        p = new_pages(1)
+        runs.append((p * bs + int(torch.randint(0, bs, (1,), generator=gen)), 1))
+    runs.append((-1, 1))
+    for length in (48, 7, 512):
+        p = new_pages((length + bs - 1) // bs)
+        runs.append((p * bs, length))
+    order = torch.randperm(page, generator=gen)  # the pages are handed out in random order
+    slots = []
+    for first, length in runs:
+        if first < 0:
+            slots.append(torch.full((length,), -1, dtype=torch.int64))
+            continue
+        s = first + torch.arange(length)
+        slots.append(order[s // bs] * bs + s % bs)
+    return torch.cat(slots), page
+
+
+@pytest.mark.parametrize("bs", [16, 64, 1024])
+@pytest.mark.parametrize("mode", ["token", "tensor", "bf16"])
+def test_cache_write_of_many_tokens_matches_the_host_quantiser(cuda, mode, bs):
+    """Thousands of tokens in one call take the kernel that writes runs of tokens 16 at a time: every run shape
+    (aligned, offset, shorter than 16, crossing pages, scattered, padding) must give the bytes and scales of the
+    host-side quantiser, and must leave every other slot of the cache untouched."""
+    import triton_op_amd as T
+
+    h, d = 3, 128
+    g = torch.Generator().manual_seed(100 + bs)
+    slots, nblk = _prefill_like_slots(bs, g)
+    toks = slots.numel()
+    assert toks >= 2048
+    live = slots >= 0
+    key = torch.randn(toks, h, d, generator=g).to(torch.bfloat16)
+    value = torch.randn(toks, h, d, generator=g).to(torch.bfloat16)
+    key[7, 1] = 0  # an all-zero row: scale 1, bytes 0
+    if mode == "token":  # rows of extreme magnitude: scales outside and inside the range of the short division
+        key[11, 0] *= 1e30
+        value[12, 2] *= 1e-30
+        key[13, 1] *= 1e-20
+        key[13, 1, 5] = 1e20
+        value[14, 0] *= 1e9
+        key[15, 2] *= 1e-9
+    fill = 0.5  # what the cache holds before the call
+    k_tok = torch.full((nblk, bs, h, d), fill, dtype=torch.bfloat16)
+    v_tok = torch.full((nblk, bs, h, d), fill, dtype=torch.bfloat16)
+    k_tok.view(-1, h, d)[slots[live]] = key[live]
+    v_tok.view(-1, h, d)[slots[live]] = value[live]
+    kc16, vc16 = L.tokens_to_key_cache(k_tok), L.tokens_to_value_cache(v_tok)
+    written = torch.zeros(nblk * bs, dtype=torch.bool)
+    written[slots[live]] = True
+    wk = written.view(nblk, 1, 1, bs, 1)
+    wv = written.view(nblk, 1, 1, bs)
+    if mode == "bf16":
+        kref, vref = kc16, vc16
+        kc, vc = torch.full_like(kc16, fill).to(cuda), torch.full_like(vc16, fill).to(cuda)
+        ks = vs = None
+    else:
+        if mode == "token":
+            kref, ksr, vref, vsr = L.quantize_kv_cache_per_token(kc16, vc16)
+            ks = torch.full((nblk, h, bs, 1), 7.0, device=cuda)
+            vs = torch.full((nblk, h, bs, 1), 7.0, device=cuda)
+        else:
+            ksr = (key.float().abs().max() / 448.0).to(torch.float32)
+            vsr = (value.float().abs().max() / 448.0).to(torch.float32)
+            kref = L.tokens_to_key_cache((k_tok.float() / ksr).to(torch.float8_e4m3fn))
+            vref = L.tokens_to_value_cache((v_tok.float() / vsr).to(torch.float8_e4m3fn))
+            ks, vs = ksr.to(cuda), vsr.to(cuda)
+        kc = torch.full(kref.shape, 0x55, dtype=torch.uint8, device=cuda).view(torch.float8_e4m3fn)
+        vc = torch.full(vref.shape, 0x55, dtype=torch.uint8, device=cuda).view(torch.float8_e4m3fn)
+    T.kv_cache_write(key.to(cuda), value.to(cuda), kc, vc, slots.to(cuda), ks, vs)
+    torch.cuda.synchronize()
+    view = torch.uint8 if mode != "bf16" else torch.int16
+    kgot, vgot = kc.cpu().view(view), vc.cpu().view(view)
+    kexp, vexp = kref.view(view).clone(), vref.view(view).clone()
+    before = 0x55 if mode != "bf16" else int(torch.tensor(fill, dtype=torch.bfloat16).view(torch.int16))
+    kexp[~wk.expand_as(kexp)] = before
+    vexp[~wv.expand_as(vexp)] = before
+    assert torch.equal(kgot, kexp)
+    assert torch.equal(vgot, vexp)
+    if mode == "token":
+        w = written.view(nblk, 1, bs, 1).expand(nblk, h, bs, 1)
+        assert torch.equal(ks.cpu()[w], ksr[w]) and torch.equal(vs.cpu()[w], vsr[w])
+        assert bool((ks.cpu()[~w] == 7.0).all()) and bool((vs.cpu()[~w] == 7.0).all())
+        assert float(ks[int(slots[7]) // bs, 1, int(slots[7]) % bs, 0]) == 1.0

@@ -22,16 +22,12 @@ __device__ __forceinline__ uint8_t f32_to_fp8(float x) {
   return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false) & 0xff);
 }
 
-// ---- append: one wave per (token, kv head); lane l owns head dims 2l, 2l+1 --------------------------------
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// ---- one (token, kv head) by one wave; lane l owns head dims 2l, 2l+1 ----------------------------------------
 template <bool TO_FP8>
-__global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs a) {
-  const int lane = threadIdx.x & 63;
-  const long long item = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= (long long)a.num_tokens * a.num_kv_heads) return;
-  const int h = (int)(item % a.num_kv_heads);
-  const long long t = item / a.num_kv_heads;
-  const long long slot = a.slot_mapping[t];
-  if (slot < 0) return;  // padding token
+__device__ __forceinline__ void write_token(const PaKvWriteArgs& a, long long t, int h, long long slot, int lane) {
   const long long block = slot / a.block_size;
   const int off = (int)(slot - block * a.block_size);
   const int bs = a.block_size;
@@ -46,7 +42,6 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs
     uint16_t* vc = (uint16_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
     vc[(int64_t)d0 * bs + off] = (uint16_t)(vraw & 0xffffu);
     vc[(int64_t)(d0 + 1) * bs + off] = (uint16_t)(vraw >> 16);
-    return;
   } else {
     const float k0 = bf16_to_f32(kraw & 0xffffu), k1 = bf16_to_f32(kraw >> 16);
     const float v0 = bf16_to_f32(vraw & 0xffffu), v1 = bf16_to_f32(vraw >> 16);
@@ -81,6 +76,307 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs
   }
 }
 
+// ---- append, a few tokens (decode): one wave per (token, kv head) ------------------------------------------------
+template <bool TO_FP8>
+__global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs a) {
+  const int lane = threadIdx.x & 63;
+  const long long item = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long long)a.num_tokens * a.num_kv_heads) return;
+  const int h = (int)(item % a.num_kv_heads);
+  const long long t = item / a.num_kv_heads;
+  const long long slot = a.slot_mapping[t];
+  if (slot < 0) return;  // padding token
+  write_token<TO_FP8>(a, t, h, slot, lane);
+}
+
+// ---- append, many tokens (prefill): one workgroup per (16 tokens, up to 4 kv heads) -----------------------------
+// Written token by token the V cache takes 128 separate one-byte stores per token and head (a token is one
+// byte of every head dim's row) and the K cache 2-byte ones; prefill appends runs of tokens to consecutive slots,
+// so here a GROUP, a run of up to 16 tokens that fill consecutive slots of one 16-slot aligned segment of a
+// page, is quantised together: 256 threads load the rows 16 bytes at a time, K leaves as 16-byte (token, chunk)
+// cells, and V is turned through LDS so that each head dim's row gets its 16 tokens in one 16-byte store.
+// A workgroup owns the groups that START among its 16 tokens (a group may reach into the next workgroup's
+// tokens, which then skips them); with more than four groups among its tokens (scattered slots) it writes its
+// tokens one by one like the kernel above.
+// lane exchanges inside a row of 16 lanes on the vector ALU (DPP), not through the LDS crossbar
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+constexpr int kDppSwap1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppSwap2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i of each 8
+constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i
+// maximum over the 16 lanes of a row (the operation commutes, so mirrors do for the last two steps)
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppSwap1>(__float_as_uint(v))));
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppSwap2>(__float_as_uint(v))));
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppHalfMirror>(__float_as_uint(v))));
+  v = fmaxf(v, __uint_as_float(dpp_u32<kDppMirror>(__float_as_uint(v))));
+  return v;
+}
+
+// Eight values of one row divided by the row's scale and rounded to e4m3fn, four bytes per word.
+// x / s must be the correctly rounded float32 quotient (what the host-side formula computes).  A float division
+// expands to a reciprocal, one correction of it and two corrections of the quotient; with one divisor for the
+// whole row the reciprocal part is done once and a value costs five instructions instead of ten.  That short
+// form is exact while nothing over- or underflows on the way: it is used for scales within 2^-40 .. 2^40 and
+// values below 2^80 (a quotient too small for its residual to be exact is far below the smallest FP8 value and
+// rounds to zero either way); anything else takes the full division.
+__device__ __forceinline__ void quantize8(const float (&x)[8], float s, u32x2& out) {
+  float q[8];
+  float xmax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) xmax = fmaxf(xmax, fabsf(x[e]));
+  const float as = fabsf(s);
+  if (as > 0x1p-40f && as < 0x1p40f && xmax < 0x1p80f) {
+    const float r0 = __builtin_amdgcn_rcpf(s);
+    const float r = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.f), r0, r0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float q0 = x[e] * r;
+      const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, x[e]), r, q0);
+      q[e] = __builtin_fmaf(__builtin_fmaf(-s, q1, x[e]), r, q1);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q[e] = __fdiv_rn(x[e], s);
+  }
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    // clamp like fminf(fmaxf(x, -448), 448) (a NaN becomes -448), then two conversions of two values each
+    const float c0 = __builtin_amdgcn_fmed3f(q[4 * w], -kFp8Max, kFp8Max), c1 = __builtin_amdgcn_fmed3f(q[4 * w + 1], -kFp8Max, kFp8Max);
+    const float c2 = __builtin_amdgcn_fmed3f(q[4 * w + 2], -kFp8Max, kFp8Max), c3 = __builtin_amdgcn_fmed3f(q[4 * w + 3], -kFp8Max, kFp8Max);
+    int word = __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false);
+    word = __builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, word, true);
+    out[w] = (uint32_t)word;
+  }
+}
+
+constexpr int kHeadsPerWorkgroup = 4;  // kv heads one workgroup of the tile kernel walks, their rows all requested first
+
+// one kv head of a group: kr, vr are this thread's 16 bytes of the token's K and V row
+template <bool TO_FP8>
+__device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, long long block, int off0, int h, int tid,
+                                                 u32x4 kr, u32x4 vr, uint8_t (*s_v)[256]) {
+  const int bs = a.block_size;
+  const int tk = tid >> 4, c = tid & 15;  // token of the group; 16-byte piece of its row (head dims 8c..8c+7)
+  const bool on = tk < n;
+  if constexpr (!TO_FP8) {
+    if (on) {
+      // K: the 16 bytes are one (chunk, token) cell of the cache as they are
+      uint16_t* kc = (uint16_t*)a.key_cache + block * a.stride_kc_b + h * a.stride_kc_h;
+      *reinterpret_cast<u32x4*>(kc + ((int64_t)c * bs + off0 + tk) * 8) = kr;
+      *reinterpret_cast<u32x4*>(&s_v[tk][16 * c]) = vr;
+    }
+    __syncthreads();
+    if (tid < 128) {  // thread = head dim: its n tokens are 2n consecutive bytes of the dim's row
+      uint16_t* vc = (uint16_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h + (int64_t)tid * bs + off0;
+      if (n == 16 && (off0 & 7) == 0) {
+        u32x4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo[e] = (uint32_t)*reinterpret_cast<const uint16_t*>(&s_v[2 * e][2 * tid]) |
+                  ((uint32_t)*reinterpret_cast<const uint16_t*>(&s_v[2 * e + 1][2 * tid]) << 16);
+          hi[e] = (uint32_t)*reinterpret_cast<const uint16_t*>(&s_v[8 + 2 * e][2 * tid]) |
+                  ((uint32_t)*reinterpret_cast<const uint16_t*>(&s_v[9 + 2 * e][2 * tid]) << 16);
+        }
+        *reinterpret_cast<u32x4*>(vc) = lo;
+        *reinterpret_cast<u32x4*>(vc + 8) = hi;
+      } else {
+        for (int k = 0; k < n; ++k) vc[k] = *reinterpret_cast<const uint16_t*>(&s_v[k][2 * tid]);
+      }
+    }
+    __syncthreads();  // s_v is free for the next group
+  } else {
+    float kf[8], vf[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      kf[2 * e] = bf16_to_f32(kr[e] & 0xffffu);
+      kf[2 * e + 1] = bf16_to_f32(kr[e] >> 16);
+      vf[2 * e] = bf16_to_f32(vr[e] & 0xffffu);
+      vf[2 * e + 1] = bf16_to_f32(vr[e] >> 16);
+    }
+    float ks, vs;
+    if (a.kv_quant_mode == PA_QUANT_PER_TOKEN) {
+      float ka = 0.f, va = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ka = fmaxf(ka, fabsf(kf[e]));
+        va = fmaxf(va, fabsf(vf[e]));
+      }
+      ka = row16_max(ka);  // the 16 lanes of a token
+      va = row16_max(va);
+      ks = ka > 0.f ? __fdiv_rn(ka, kFp8Max) : 1.f;
+      vs = va > 0.f ? __fdiv_rn(va, kFp8Max) : 1.f;
+      if (on && c == 0) {
+        const int64_t so = block * a.stride_scale_b + h * a.stride_scale_h + off0 + tk;
+        a.key_scale[so] = ks;
+        a.value_scale[so] = vs;
+      }
+    } else if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
+      ks = a.key_scale[0];
+      vs = a.value_scale[0];
+    } else {
+      ks = vs = 1.f;
+    }
+    u32x2 kq, vq;
+    quantize8(kf, ks, kq);
+    quantize8(vf, vs, vq);
+    // K: lanes c, c+1 hold the two halves of one 16-byte (chunk, token) cell; the even one stores it
+    const uint32_t p0 = dpp_u32<kDppSwap1>(kq[0]), p1 = dpp_u32<kDppSwap1>(kq[1]);
+    if (on) {
+      if ((c & 1) == 0) {
+        uint8_t* kc = (uint8_t*)a.key_cache + block * a.stride_kc_b + h * a.stride_kc_h;
+        *reinterpret_cast<u32x4*>(kc + ((int64_t)(c >> 1) * bs + off0 + tk) * 16) = u32x4{kq[0], kq[1], p0, p1};
+      }
+      *reinterpret_cast<u32x2*>(&s_v[tk][8 * c]) = vq;
+    }
+    __syncthreads();
+    if (tid < 128) {  // thread = head dim: its n tokens are n consecutive bytes of the dim's row
+      uint8_t* vc = (uint8_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h + (int64_t)tid * bs + off0;
+      if (n == 16 && (off0 & 15) == 0) {
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = (uint32_t)s_v[4 * e][tid] | ((uint32_t)s_v[4 * e + 1][tid] << 8) | ((uint32_t)s_v[4 * e + 2][tid] << 16) |
+                 ((uint32_t)s_v[4 * e + 3][tid] << 24);
+        *reinterpret_cast<u32x4*>(vc) = o;
+      } else {
+        for (int k = 0; k < n; ++k) vc[k] = s_v[k][tid];
+      }
+    }
+    __syncthreads();  // s_v is free for the next group
+  }
+}
+
+// a group of n tokens from token t_first on, landing at slot0 .. slot0 + n - 1, for kv heads h0 .. h0 + nh - 1
+template <bool TO_FP8>
+__device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_first, int n, long long slot0, int h0, int nh,
+                                            int tid, uint8_t (*s_v)[256]) {
+  const long long block = slot0 / a.block_size;
+  const int off0 = (int)(slot0 - block * a.block_size);
+  const int tk = tid >> 4, c = tid & 15;
+  u32x4 kr[kHeadsPerWorkgroup], vr[kHeadsPerWorkgroup];
+#pragma unroll
+  for (int i = 0; i < kHeadsPerWorkgroup; ++i) {
+    kr[i] = vr[i] = u32x4{0, 0, 0, 0};
+    if (tk < n && i < nh) {  // the rows are read once: non-temporal
+      const long long t = t_first + tk;
+      kr[i] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4*>((const uint16_t*)a.key + t * a.stride_k_t + (h0 + i) * a.stride_k_h + 8 * c));
+      vr[i] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4*>((const uint16_t*)a.value + t * a.stride_v_t + (h0 + i) * a.stride_v_h + 8 * c));
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kHeadsPerWorkgroup; ++i) {
+    if (i < nh) write_group_head<TO_FP8>(a, n, block, off0, h0 + i, tid, kr[i], vr[i], s_v);
+  }
+}
+
+// With pages of more than 16 tokens the groups of neighbouring 16-token windows write neighbouring 16-byte
+// pieces of the same 128-byte lines of the V cache, and the pieces only merge into whole lines if they pass
+// through the same L2 close together.  Workgroups go to the eight XCDs (each with an L2 of its own) round robin
+// in id order, so with `regroup` set the window a workgroup takes is chosen such that the eight windows of a
+// 128-token stretch are the next eight workgroups of ONE XCD.  The grid is then a multiple of 64 windows.
+template <bool TO_FP8>
+__global__ __launch_bounds__(256) void kv_cache_write_tile_kernel(const PaKvWriteArgs a, const int regroup) {
+  __shared__ long long s_slot[33];  // slots of tokens t0-1 .. t0+31
+  __shared__ __attribute__((aligned(16))) uint8_t s_v[16][256];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  long long window = blockIdx.x;
+  if (regroup) {
+    const long long q = window >> 3, xcd = window & 7;
+    window = (((q >> 3) << 3) + xcd) * 8 + (q & 7);
+  }
+  const long long t0 = window * 16;
+  if (t0 >= a.num_tokens) return;
+  const int h0 = blockIdx.y * kHeadsPerWorkgroup;
+  const int nh = min(kHeadsPerWorkgroup, a.num_kv_heads - h0);
+  if (tid < 33) {
+    const long long t = t0 - 1 + tid;
+    s_slot[tid] = (t >= 0 && t < a.num_tokens) ? a.slot_mapping[t] : -1;
+  }
+  __syncthreads();
+  // bit j of `starts`: token t0+j is live and does not continue its predecessor's run inside a 16-slot segment;
+  // bit j of `breaks`: a group that reaches token t0+j ends before it.  Every wave computes both.
+  bool is_start = false, is_live = false;
+  if (lane < 32) {
+    const long long cur = s_slot[lane + 1], prev = s_slot[lane];
+    is_live = cur >= 0;
+    is_start = is_live && (prev < 0 || cur != prev + 1 || (cur & 15) == 0);
+  }
+  const uint64_t starts = __builtin_amdgcn_ballot_w64(is_start);
+  const uint64_t breaks = starts | (~__builtin_amdgcn_ballot_w64(is_live) & 0xffffffffull) | (1ull << 32);
+  uint32_t own = (uint32_t)starts & 0xffffu;  // the groups that start among this workgroup's 16 tokens
+  if (own == 0) return;
+  if (__builtin_popcount(own) > 4) {
+    // scattered slots: token by token, the waves taking turns.  Token t0+k is this workgroup's if the last
+    // start at or before it is among the first 16 tokens.
+    const int wave = tid >> 6;
+    for (int k = wave; k < 32; k += 4) {
+      const uint64_t upto = starts & ((2ull << k) - 1);
+      if (((breaks >> k) & 1) && !((starts >> k) & 1)) continue;  // not live
+      if (upto == 0 || (63 - __builtin_clzll(upto)) >= 16) continue;
+      for (int i = 0; i < nh; ++i) write_token<TO_FP8>(a, t0 + k, h0 + i, s_slot[k + 1], lane);
+    }
+    return;
+  }
+  while (own) {
+    const int j = __builtin_ctz(own);
+    own &= own - 1;
+    const int n = __builtin_ctzll(breaks >> (j + 1)) + 1;
+    write_group<TO_FP8>(a, t0 + j, n, s_slot[j + 1], h0, nh, tid, s_v);
+  }
+}
+
+// ---- whole cache, per token, 16 tokens of one (block, kv head) per workgroup ------------------------------------
+// The 16-bit cache (x = 8) is read in its own layout, 16 bytes per thread: K cells as they lie, V rows (8 tokens of
+// one head dim) through LDS into the per-token form the append kernel works on; from there on it IS the append of
+// a full group.  a.key / a.value are the 16-bit caches here.  Windows of one page are regrouped by XCD as above.
+__global__ __launch_bounds__(256) void quantize_kv_cache_tile_kernel(const PaKvWriteArgs a, const long long num_windows,
+                                                                    const int regroup) {
+  __shared__ __attribute__((aligned(16))) uint8_t s_v[16][256];
+  __shared__ uint32_t s_in[128][9];  // V rows of the window: 16 bf16 tokens per head dim, padded to 9 words
+  const int tid = threadIdx.x;
+  long long window = blockIdx.x;
+  if (regroup) {
+    const long long q = window >> 3, xcd = window & 7;
+    window = (((q >> 3) << 3) + xcd) * 8 + (q & 7);
+  }
+  if (window >= num_windows) return;
+  const int bs = a.block_size;
+  const int wins_per_page = bs >> 4;
+  const long long bh = window / wins_per_page;  // (block, head)
+  const int tok0 = (int)(window - bh * wins_per_page) * 16;
+  const long long block = bh / a.num_kv_heads;
+  const int h = (int)(bh - block * a.num_kv_heads);
+  const uint16_t* kin = (const uint16_t*)a.key + bh * 128 * bs;    // [16 chunks][bs][8]
+  const uint16_t* vin = (const uint16_t*)a.value + bh * 128 * bs;  // [128][bs]
+  const int tk = tid >> 4, c = tid & 15;
+  const u32x4 kr = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kin + ((int64_t)c * bs + tok0 + tk) * 8));
+  {
+    const int d = tid >> 1, half = tid & 1;
+    // with more than one window per page a window reads a piece of each 128-byte line and its neighbours (same
+    // XCD) the rest: those lines must stay in L2, so only whole-page windows read V non-temporally
+    const u32x4* vp = reinterpret_cast<const u32x4*>(vin + (int64_t)d * bs + tok0 + 8 * half);
+    const u32x4 v = regroup ? *vp : __builtin_nontemporal_load(vp);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s_in[d][4 * half + e] = v[e];
+  }
+  __syncthreads();
+  u32x4 vr;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {  // head dims 8c + 2e, 8c + 2e + 1 of token tk
+    const uint32_t w0 = s_in[8 * c + 2 * e][tk >> 1], w1 = s_in[8 * c + 2 * e + 1][tk >> 1];
+    const int sh = 16 * (tk & 1);
+    vr[e] = ((w0 >> sh) & 0xffffu) | (((w1 >> sh) & 0xffffu) << 16);
+  }
+  write_group_head<true>(a, 16, block, tok0, h, tid, kr, vr, s_v);
+}
+
 // ---- whole cache, per token: one thread per (block, kv head, token) -------------------------------------------
 // Reads the 16-bit cache in its own layout (x = 8) and writes the FP8 cache (x = 16) and the scales.
 __global__ __launch_bounds__(256) void quantize_kv_cache_kernel(const uint16_t* __restrict__ kin, const uint16_t* __restrict__ vin,
@@ -93,7 +389,6 @@ __global__ __launch_bounds__(256) void quantize_kv_cache_kernel(const uint16_t* 
   const int tok = (int)(idx - bh * bs);
   const uint16_t* kp = kin + bh * 128 * bs;  // [16 chunks][bs][8]
   const uint16_t* vp = vin + bh * 128 * bs;  // [128][bs]
-  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
   float ka = 0.f, va = 0.f;
   u32x4 kc[16];
 #pragma unroll
@@ -159,10 +454,27 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
   const long long blocks = (items + 3) / 4;
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-  if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
+  // Many tokens (prefill) go 16 at a time when the rows can be read 16 bytes at a time; a few tokens (decode)
+  // get one wave per (token, head) each, which has more of the GPU working on them.
+  const bool rows_16b = a->stride_k_t % 8 == 0 && a->stride_k_h % 8 == 0 && a->stride_v_t % 8 == 0 && a->stride_v_h % 8 == 0 &&
+                        ((reinterpret_cast<uintptr_t>(a->key) | reinterpret_cast<uintptr_t>(a->value)) & 15) == 0 &&
+                        ((reinterpret_cast<uintptr_t>(a->key_cache) | reinterpret_cast<uintptr_t>(a->value_cache)) & 15) == 0 &&
+                        a->stride_kc_b % 16 == 0 && a->stride_kc_h % 16 == 0 && a->stride_vc_b % 16 == 0 && a->stride_vc_h % 16 == 0 &&
+                        a->block_size % 16 == 0;
+  if (rows_16b && a->num_tokens >= 2048 && a->num_kv_heads <= 65535) {
+    const int regroup = a->block_size > 16;
+    long long windows = (a->num_tokens + 15) / 16;
+    if (regroup) windows = (windows + 63) / 64 * 64;
+    const dim3 grid((unsigned)windows, (unsigned)((a->num_kv_heads + kHeadsPerWorkgroup - 1) / kHeadsPerWorkgroup));
+    if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
+      hipLaunchKernelGGL(kv_cache_write_tile_kernel<true>, grid, dim3(256), 0, stream, *a, regroup);
+    else
+      hipLaunchKernelGGL(kv_cache_write_tile_kernel<false>, grid, dim3(256), 0, stream, *a, regroup);
+  } else if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN) {
     hipLaunchKernelGGL(kv_cache_write_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
-  else
+  } else {
     hipLaunchKernelGGL(kv_cache_write_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error_kv = (int)e;
@@ -179,11 +491,39 @@ int pa_quantize_kv_cache(const void* key_cache_bf16, const void* value_cache_bf1
   if (num_blocks <= 0 || num_kv_heads <= 0 || block_size <= 0) return PA_ERR_BAD_SHAPE;
   if (head_size != 128) return PA_ERR_UNSUPPORTED;
   const long long n = (long long)num_blocks * num_kv_heads * block_size;
-  const long long blocks = (n + 255) / 256;
-  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(quantize_kv_cache_kernel, dim3((unsigned)blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(hip_stream),
-                     (const uint16_t*)key_cache_bf16, (const uint16_t*)value_cache_bf16, (uint8_t*)key_cache_fp8,
-                     (uint8_t*)value_cache_fp8, key_scale, value_scale, (long long)num_blocks * num_kv_heads, block_size);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(key_cache_bf16) | reinterpret_cast<uintptr_t>(value_cache_bf16) |
+                         reinterpret_cast<uintptr_t>(key_cache_fp8) | reinterpret_cast<uintptr_t>(value_cache_fp8)) & 15) == 0;
+  if (aligned && block_size % 16 == 0) {
+    PaKvWriteArgs a = {};
+    a.struct_size = sizeof(PaKvWriteArgs);
+    a.key = key_cache_bf16;
+    a.value = value_cache_bf16;
+    a.key_cache = key_cache_fp8;
+    a.value_cache = value_cache_fp8;
+    a.key_scale = key_scale;
+    a.value_scale = value_scale;
+    a.num_kv_heads = num_kv_heads;
+    a.head_size = head_size;
+    a.block_size = block_size;
+    a.cache_dtype = PA_DTYPE_FP8_E4M3FN;
+    a.kv_quant_mode = PA_QUANT_PER_TOKEN;
+    a.stride_kc_h = a.stride_vc_h = (int64_t)head_size * block_size;
+    a.stride_kc_b = a.stride_vc_b = a.stride_kc_h * num_kv_heads;
+    a.stride_scale_h = block_size;
+    a.stride_scale_b = (int64_t)block_size * num_kv_heads;
+    const long long num_windows = n / 16;
+    const int regroup = block_size > 16;
+    const long long grid = regroup ? (num_windows + 63) / 64 * 64 : num_windows;
+    if (grid > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(quantize_kv_cache_tile_kernel, dim3((unsigned)grid), dim3(256), 0, stream, a, num_windows, regroup);
+  } else {
+    const long long blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(quantize_kv_cache_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       (const uint16_t*)key_cache_bf16, (const uint16_t*)value_cache_bf16, (uint8_t*)key_cache_fp8,
+                       (uint8_t*)value_cache_fp8, key_scale, value_scale, (long long)num_blocks * num_kv_heads, block_size);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     g_last_hip_error_kv = (int)e;
