@@ -171,6 +171,9 @@ int pa_decode(const PaDecodeArgs* args, void* hip_stream);
  * tensor (the given scales are read), or cast as they are.  The reference has this step only as an
  * offline whole-cache routine, quantize_kv_cache_symmetric (test_pa_mtp.py:294-369, over
  * aiter.pertoken_quant), which pa_quantize_kv_cache below replaces directly.
+ * Calls with 2048 tokens or more whose rows, caches and strides are 16-byte aligned (and block_size a
+ * multiple of 16) are written in runs of up to 16 tokens that land in consecutive slots; any slot_mapping is
+ * valid (runs are found on the device), the bytes written are the same either way.
  */
 typedef struct PaKvWriteArgs {
   uint32_t struct_size; /* = sizeof(PaKvWriteArgs) */
