@@ -182,7 +182,7 @@ typedef struct PaKvWriteArgs {
   const void* value;           /* bf16 [num_tokens, Hkv, D] */
   const int64_t* slot_mapping; /* [num_tokens] */
   void* key_cache;             /* [blocks, Hkv, D/x, bs, x] */
-  void* value_cache;           /* [blocks, Hkv, D, bs] */
+  void* value_cache;           /* [blocks, Hkv, D, bs], or [blocks, Hkv, bs/x, D, x] with v_transposed */
   float* key_scale;            /* per token: [blocks, Hkv, bs, 1] written; per tensor: 1 value read */
   float* value_scale;
   int64_t num_tokens;
@@ -191,7 +191,7 @@ typedef struct PaKvWriteArgs {
   int32_t block_size;
   int32_t cache_dtype;         /* PA_DTYPE_* */
   int32_t kv_quant_mode;       /* PA_QUANT_* */
-  int32_t reserved1;
+  int32_t v_transposed;        /* 0: value_cache [.., D, bs]; 1: [.., bs/x, D, x] (shuffle_value_cache_layout, test_pa_mtp.py:472-497) */
   int64_t stride_k_t, stride_k_h, stride_v_t, stride_v_h; /* elements; last dim contiguous */
   int64_t stride_kc_b, stride_kc_h, stride_vc_b, stride_vc_h; /* cache block / head strides; inner dims dense */
   int64_t stride_scale_b, stride_scale_h;

@@ -27,8 +27,9 @@ def test_quantize_whole_cache_matches_torch_bit_for_bit(cuda, bs, nblk, h):
     assert torch.equal(vsf.cpu(), vs_ref.permute(1, 0, 2, 3).reshape(h, nblk * bs))
 
 
+@pytest.mark.parametrize("trans_v", [False, True], ids=["plainV", "transV"])
 @pytest.mark.parametrize("mode", ["token", "tensor", "bf16"])
-def test_cache_write_then_decode(cuda, mode):
+def test_cache_write_then_decode(cuda, mode, trans_v):
     """Tokens appended through kv_cache_write (in two calls, scattered slots, one padding token) give the same
     cache bytes as the host-side quantiser, and the decode op reads them back correctly."""
     import triton_op_amd as T
@@ -68,6 +69,8 @@ def test_cache_write_then_decode(cuda, mode):
             kref = L.tokens_to_key_cache((k_tok.float() / ksr).to(torch.float8_e4m3fn))
             vref = L.tokens_to_value_cache((v_tok.float() / vsr).to(torch.float8_e4m3fn))
             ks, vs = ksr.to(dev), vsr.to(dev)
+    if trans_v:  # the kernel writes (and the decode op reads) the transposed V layout
+        vc = L.shuffle_value_cache_layout(vc)
     # append in two calls; the second carries a padding token (slot -1)
     cut = 90
     T.kv_cache_write(key[:cut].to(dev), value[:cut].to(dev), kc, vc, slots[:cut].to(dev), ks, vs)
@@ -78,7 +81,8 @@ def test_cache_write_then_decode(cuda, mode):
     torch.cuda.synchronize()
     view = torch.uint8 if mode != "bf16" else torch.int16
     assert torch.equal(kc.cpu().view(view), kref.view(view))
-    assert torch.equal(vc.cpu().view(view), vref.view(view))
+    vplain = L.unshuffle_value_cache_layout(vc) if trans_v else vc
+    assert torch.equal(vplain.cpu().view(view), vref.view(view))
     if mode == "token":
         live = torch.zeros(nblk * bs, dtype=torch.bool)
         live[slots] = True
@@ -132,9 +136,10 @@ def _prefill_like_slots(bs, gen):
     return torch.cat(slots), page
 
 
+@pytest.mark.parametrize("trans_v", [False, True], ids=["plainV", "transV"])
 @pytest.mark.parametrize("bs", [16, 64, 1024])
 @pytest.mark.parametrize("mode", ["token", "tensor", "bf16"])
-def test_cache_write_of_many_tokens_matches_the_host_quantiser(cuda, mode, bs):
+def test_cache_write_of_many_tokens_matches_the_host_quantiser(cuda, mode, bs, trans_v):
     """Thousands of tokens in one call take the kernel that writes runs of tokens 16 at a time: every run shape
     (aligned, offset, shorter than 16, crossing pages, scattered, padding) must give the bytes and scales of the
     host-side quantiser, and must leave every other slot of the cache untouched."""
@@ -183,8 +188,12 @@ def test_cache_write_of_many_tokens_matches_the_host_quantiser(cuda, mode, bs):
             ks, vs = ksr.to(cuda), vsr.to(cuda)
         kc = torch.full(kref.shape, 0x55, dtype=torch.uint8, device=cuda).view(torch.float8_e4m3fn)
         vc = torch.full(vref.shape, 0x55, dtype=torch.uint8, device=cuda).view(torch.float8_e4m3fn)
+    if trans_v:  # the kernel writes the transposed V layout; it is turned back for the comparison
+        vc = L.shuffle_value_cache_layout(vc)
     T.kv_cache_write(key.to(cuda), value.to(cuda), kc, vc, slots.to(cuda), ks, vs)
     torch.cuda.synchronize()
+    if trans_v:
+        vc = L.unshuffle_value_cache_layout(vc)
     view = torch.uint8 if mode != "bf16" else torch.int16
     kgot, vgot = kc.cpu().view(view), vc.cpu().view(view)
     kexp, vexp = kref.view(view).clone(), vref.view(view).clone()

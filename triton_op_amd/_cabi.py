@@ -59,7 +59,7 @@ class PaKvWriteArgs(C.Structure):
         [("struct_size", C.c_uint32), ("reserved0", C.c_int32)]
         + [(n, C.c_void_p) for n in ("key", "value", "slot_mapping", "key_cache", "value_cache", "key_scale", "value_scale")]
         + [("num_tokens", C.c_int64)]
-        + [(n, C.c_int32) for n in ("num_kv_heads", "head_size", "block_size", "cache_dtype", "kv_quant_mode", "reserved1")]
+        + [(n, C.c_int32) for n in ("num_kv_heads", "head_size", "block_size", "cache_dtype", "kv_quant_mode", "v_transposed")]
         + [(n, C.c_int64) for n in (
             "stride_k_t", "stride_k_h", "stride_v_t", "stride_v_h", "stride_kc_b", "stride_kc_h", "stride_vc_b",
             "stride_vc_h", "stride_scale_b", "stride_scale_h")]

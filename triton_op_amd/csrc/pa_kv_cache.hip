@@ -1,6 +1,6 @@
 // KV-cache write and quantisation kernels for the paged layouts the decode kernels read:
 //   key_cache   [blocks, Hkv, D/x, bs, x]     x = 16 / sizeof(element)
-//   value_cache [blocks, Hkv, D, bs]
+//   value_cache [blocks, Hkv, D, bs], or transposed [blocks, Hkv, bs/x, D, x]
 //   scales      [blocks, Hkv, bs, 1] f32 (one per token and kv head) or one f32 per tensor
 // FP8 is OCP e4m3fn.  Quantisation is symmetric: scale = amax / 448 (1 for an all-zero row),
 // q = round_to_nearest_even(x / scale), both with IEEE division so the bytes match a float32 host
@@ -25,6 +25,13 @@ __device__ __forceinline__ uint8_t f32_to_fp8(float x) {
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
+// element index of (head dim d, token offset off) inside one (block, head) of the V cache: rows of block_size
+// tokens per head dim, or, transposed, tiles of X tokens (X = 16 / element size) with the head dims inside a tile
+template <int X>
+__device__ __forceinline__ int64_t v_index(const PaKvWriteArgs& a, int d, int off) {
+  return a.v_transposed ? ((int64_t)(off / X) * 128 + d) * X + off % X : (int64_t)d * a.block_size + off;
+}
+
 // ---- one (token, kv head) by one wave; lane l owns head dims 2l, 2l+1 ----------------------------------------
 template <bool TO_FP8>
 __device__ __forceinline__ void write_token(const PaKvWriteArgs& a, long long t, int h, long long slot, int lane) {
@@ -40,8 +47,8 @@ __device__ __forceinline__ void write_token(const PaKvWriteArgs& a, long long t,
     uint16_t* kc = (uint16_t*)a.key_cache + block * a.stride_kc_b + h * a.stride_kc_h;
     *reinterpret_cast<uint32_t*>(kc + (int64_t)(d0 / 8) * bs * 8 + off * 8 + d0 % 8) = kraw;
     uint16_t* vc = (uint16_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
-    vc[(int64_t)d0 * bs + off] = (uint16_t)(vraw & 0xffffu);
-    vc[(int64_t)(d0 + 1) * bs + off] = (uint16_t)(vraw >> 16);
+    vc[v_index<8>(a, d0, off)] = (uint16_t)(vraw & 0xffffu);
+    vc[v_index<8>(a, d0 + 1, off)] = (uint16_t)(vraw >> 16);
   } else {
     const float k0 = bf16_to_f32(kraw & 0xffffu), k1 = bf16_to_f32(kraw >> 16);
     const float v0 = bf16_to_f32(vraw & 0xffffu), v1 = bf16_to_f32(vraw >> 16);
@@ -71,8 +78,8 @@ __device__ __forceinline__ void write_token(const PaKvWriteArgs& a, long long t,
     uint8_t* kc = (uint8_t*)a.key_cache + block * a.stride_kc_b + h * a.stride_kc_h;
     *reinterpret_cast<uint16_t*>(kc + (int64_t)(d0 / 16) * bs * 16 + off * 16 + d0 % 16) = (uint16_t)(qk0 | (qk1 << 8));
     uint8_t* vc = (uint8_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
-    vc[(int64_t)d0 * bs + off] = qv0;
-    vc[(int64_t)(d0 + 1) * bs + off] = qv1;
+    vc[v_index<16>(a, d0, off)] = qv0;
+    vc[v_index<16>(a, d0 + 1, off)] = qv1;
   }
 }
 
@@ -171,7 +178,7 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
     }
     __syncthreads();
     if (tid < 128) {  // thread = head dim: its n tokens are 2n consecutive bytes of the dim's row
-      uint16_t* vc = (uint16_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h + (int64_t)tid * bs + off0;
+      uint16_t* vc = (uint16_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
       if (n == 16 && (off0 & 7) == 0) {
         u32x4 lo, hi;
 #pragma unroll
@@ -181,10 +188,10 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
           hi[e] = (uint32_t)*reinterpret_cast<const uint16_t*>(&s_v[8 + 2 * e][2 * tid]) |
                   ((uint32_t)*reinterpret_cast<const uint16_t*>(&s_v[9 + 2 * e][2 * tid]) << 16);
         }
-        *reinterpret_cast<u32x4*>(vc) = lo;
-        *reinterpret_cast<u32x4*>(vc + 8) = hi;
+        *reinterpret_cast<u32x4*>(vc + v_index<8>(a, tid, off0)) = lo;  // tokens 0..7: one 8-token tile if transposed
+        *reinterpret_cast<u32x4*>(vc + v_index<8>(a, tid, off0 + 8)) = hi;
       } else {
-        for (int k = 0; k < n; ++k) vc[k] = *reinterpret_cast<const uint16_t*>(&s_v[k][2 * tid]);
+        for (int k = 0; k < n; ++k) vc[v_index<8>(a, tid, off0 + k)] = *reinterpret_cast<const uint16_t*>(&s_v[k][2 * tid]);
       }
     }
     __syncthreads();  // s_v is free for the next group
@@ -234,16 +241,16 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
     }
     __syncthreads();
     if (tid < 128) {  // thread = head dim: its n tokens are n consecutive bytes of the dim's row
-      uint8_t* vc = (uint8_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h + (int64_t)tid * bs + off0;
+      uint8_t* vc = (uint8_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
       if (n == 16 && (off0 & 15) == 0) {
         u32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           o[e] = (uint32_t)s_v[4 * e][tid] | ((uint32_t)s_v[4 * e + 1][tid] << 8) | ((uint32_t)s_v[4 * e + 2][tid] << 16) |
                  ((uint32_t)s_v[4 * e + 3][tid] << 24);
-        *reinterpret_cast<u32x4*>(vc) = o;
+        *reinterpret_cast<u32x4*>(vc + v_index<16>(a, tid, off0)) = o;
       } else {
-        for (int k = 0; k < n; ++k) vc[k] = s_v[k][tid];
+        for (int k = 0; k < n; ++k) vc[v_index<16>(a, tid, off0 + k)] = s_v[k][tid];
       }
     }
     __syncthreads();  // s_v is free for the next group
@@ -445,6 +452,8 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
   if (a->num_tokens < 0 || a->num_kv_heads <= 0 || a->block_size <= 0) return PA_ERR_BAD_SHAPE;
   if (a->head_size != 128) return PA_ERR_UNSUPPORTED;
   if (a->cache_dtype != PA_DTYPE_BF16 && a->cache_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
+  if (a->v_transposed != 0 && a->v_transposed != 1) return PA_ERR_BAD_SHAPE;
+  if (a->v_transposed && a->block_size % (a->cache_dtype == PA_DTYPE_FP8_E4M3FN ? 16 : 8)) return PA_ERR_BAD_SHAPE;
   if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN && a->kv_quant_mode != PA_QUANT_NONE && (!a->key_scale || !a->value_scale))
     return PA_ERR_NULL_POINTER;
   if (a->cache_dtype == PA_DTYPE_BF16 && a->kv_quant_mode != PA_QUANT_NONE) return PA_ERR_UNSUPPORTED;

@@ -60,7 +60,7 @@ def kv_cache_write(
     key: torch.Tensor,           # [num_tokens, num_kv_heads, head_size] bf16
     value: torch.Tensor,
     key_cache: torch.Tensor,     # [blocks, Hkv, D/x, bs, x]  bf16 or float8_e4m3fn
-    value_cache: torch.Tensor,   # [blocks, Hkv, D, bs]
+    value_cache: torch.Tensor,   # [blocks, Hkv, D, bs], or transposed [blocks, Hkv, bs/x, D, x]
     slot_mapping: torch.Tensor,  # [num_tokens] int64, block * block_size + offset; negative = skip
     key_scale: Optional[torch.Tensor] = None,    # FP8 cache: [blocks, Hkv, bs, 1] (written) or 0-dim (read)
     value_scale: Optional[torch.Tensor] = None,
@@ -78,10 +78,17 @@ def kv_cache_write(
         raise ValueError("caches must both be bfloat16 or float8_e4m3fn")
     x = 16 // key_cache.element_size()
     bs = key_cache.shape[-2]
-    if key_cache.dim() != 5 or value_cache.dim() != 4 or tuple(key_cache.shape[1:]) != (h, d // x, bs, x) or \
-            tuple(value_cache.shape[1:]) != (h, d, bs):
-        raise ValueError("cache shapes must be [blocks, Hkv, D/x, bs, x] and [blocks, Hkv, D, bs]")
-    if key_cache[0, 0].stride() != (bs * x, x, 1) or value_cache[0, 0].stride() != (bs, 1):
+    v_transposed = value_cache.dim() == 5
+    v_inner = (bs // x, d, x) if v_transposed else (d, bs)
+    if key_cache.dim() != 5 or tuple(key_cache.shape[1:]) != (h, d // x, bs, x) or \
+            tuple(value_cache.shape[1:]) != (h,) + v_inner or (v_transposed and bs % x):
+        raise ValueError("cache shapes must be [blocks, Hkv, D/x, bs, x] and [blocks, Hkv, D, bs] "
+                         "(or [blocks, Hkv, bs/x, D, x] for the transposed V layout)")
+    v_dense = (d * x, x, 1) if v_transposed else (bs, 1)
+    def _dense(t, want):  # the stride of a dimension of size 1 means nothing
+        return all(n == 1 or st == w for n, st, w in zip(t.shape, t.stride(), want))
+
+    if not _dense(key_cache[0, 0], (bs * x, x, 1)) or not _dense(value_cache[0, 0], v_dense):
         raise ValueError("the cache dimensions inside a (block, head) must be dense")
     a = PaKvWriteArgs()
     a.struct_size = C.sizeof(PaKvWriteArgs)
@@ -106,6 +113,7 @@ def kv_cache_write(
             a.stride_scale_b, a.stride_scale_h = key_scale.stride(0), key_scale.stride(1)
         a.key_scale, a.value_scale = key_scale.data_ptr(), value_scale.data_ptr()
     a.kv_quant_mode = mode
+    a.v_transposed = 1 if v_transposed else 0
     a.stride_k_t, a.stride_k_h, a.stride_v_t, a.stride_v_h = key.stride(0), key.stride(1), value.stride(0), value.stride(1)
     a.stride_kc_b, a.stride_kc_h = key_cache.stride(0), key_cache.stride(1)
     a.stride_vc_b, a.stride_vc_h = value_cache.stride(0), value_cache.stride(1)
