@@ -26,6 +26,7 @@ There is no eager/torch implementation behind this function: without the HIP lib
 from __future__ import annotations
 
 import ctypes as C
+import functools
 from typing import Dict, Optional
 
 import torch
@@ -50,9 +51,11 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+@functools.lru_cache(maxsize=4096)
 def select_partition_size(num_seqs: int, num_kv_heads: int, rows_per_group: int, max_context_len: int,
                           block_size: int, num_cus: int = 0) -> int:
-    """The tuning layer's choice of tokens per partition (a multiple of 256)."""
+    """The tuning layer's choice of tokens per partition (a multiple of 256).  A pure function of its
+    arguments (and of the GPU's CU count when num_cus is 0), hence cached."""
     lib = _cabi.load_library()
     ps = lib.pa_decode_select_partition_size(num_seqs, num_kv_heads, rows_per_group, max(1, max_context_len),
                                              block_size, num_cus)
@@ -272,10 +275,22 @@ def plan_decode(
         max_parts = needed_parts
         shape = (num_seqs, num_kv_heads, max_parts, ge)
         # zero-filled like the reference's (:1729-1733): slots of partitions a sequence does not reach
-        # are never written or read by the kernels
-        max_logits = torch.zeros(shape, dtype=torch.float32, device=dev)
-        exp_sums = torch.zeros(shape, dtype=torch.float32, device=dev)
-        tmp_output = torch.zeros(shape + (head_size,), dtype=torch.bfloat16, device=dev)
+        # are never written or read by the kernels.  One allocation and one fill for the three buffers (and the
+        # workspace, when the caller brought none): each torch.zeros is a kernel launch and ~5 us of host time.
+        n = num_seqs * num_kv_heads * max_parts * ge
+        sizes = [4 * n, 4 * n, 2 * n * head_size]
+        if workspace is None:
+            sizes.append(int(_cabi.load_library().pa_decode_workspace_bytes(num_seqs, max_parts)))
+        offs, total = [], 0
+        for sz in sizes:
+            offs.append(total)
+            total += -(-sz // 256) * 256
+        pool = torch.zeros(total, dtype=torch.uint8, device=dev)
+        max_logits = pool[offs[0]:offs[0] + sizes[0]].view(torch.float32).view(shape)
+        exp_sums = pool[offs[1]:offs[1] + sizes[1]].view(torch.float32).view(shape)
+        tmp_output = pool[offs[2]:offs[2] + sizes[2]].view(torch.bfloat16).view(shape + (head_size,))
+        if workspace is None:
+            workspace = pool[offs[3]:offs[3] + -(-sizes[3] // 4) * 4].view(torch.int32)
 
     a = PaDecodeArgs()
     a.struct_size = C.sizeof(PaDecodeArgs)
