@@ -30,8 +30,15 @@ extern "C" {
  * several rounds of workgroups a small planning kernel lists the live (sequence, partition) items, whole
  * partitions first and the sequences' last, partial partitions by decreasing length, and the partition kernel
  * takes its items from the list (longest-first keeps the end of a ragged batch's launch busy).  The list is
- * rewritten by every call.  Calls that may overlap on the GPU need a workspace each. */
+ * rewritten by every call (unless PA_DECODE_FLAG_REUSE_ITEM_LIST says it is still good).  Calls that may overlap
+ * on the GPU need a workspace each. */
 #define PA_DECODE_WORKSPACE_BYTES 64
+/*
+ * flags: the workspace still holds the item list that an earlier call built for the SAME context_lens contents,
+ * num_seqs, max_num_partitions and partition_size (the previous layer of one decode step, say): the planning
+ * kernel is skipped (about 4.5 us).  Ignored by launches that use no item list.
+ */
+#define PA_DECODE_FLAG_REUSE_ITEM_LIST 1
 
 /* element types */
 enum { PA_DTYPE_BF16 = 0, PA_DTYPE_FP8_E4M3FN = 1 };
@@ -73,7 +80,7 @@ enum {
  */
 typedef struct PaDecodeArgs {
   uint32_t struct_size; /* = sizeof(PaDecodeArgs) */
-  int32_t reserved0;     /* 0 */
+  int32_t flags;         /* 0 or PA_DECODE_FLAG_* */
 
   void* output;
   const void* query;

@@ -356,6 +356,40 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("group,q_len,scale_mode", [(8, 1, "tensor"), (16, 3, "token")])
+def test_item_list_reused_by_the_next_layer(cuda, group, q_len, scale_mode):
+    """Two layers of one decode step share the sequence lengths and a workspace: the second is told to reuse the
+    item list the first one's planning kernel left there.  Its result must be the one it computes on its own."""
+    import triton_op_amd as T
+    from triton_op_amd import _cabi
+
+    gen = torch.Generator().manual_seed(23)
+    batch = 96
+    ctx = torch.clamp(torch.randint(1, 2600, (batch,), generator=gen, dtype=torch.int32), min=q_len)
+    kw = dict(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, scale_mode=scale_mode)
+    layers = [_make(**kw, seed=7).to(cuda), _make(**kw, seed=8).to(cuda)]
+    parts = -(-int(ctx.max()) // 256)
+    ws = torch.zeros(int(_cabi.load_library().pa_decode_workspace_bytes(batch, parts)) // 4 + 1, dtype=torch.int32, device=cuda)
+    outs = []
+    for i, g in enumerate(layers):
+        out = torch.full_like(g.query, float("nan"))
+        T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                                 q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                                 partition_size=256, workspace=ws, reuse_item_list=i > 0)
+        outs.append(out)
+    alone = torch.full_like(layers[1].query, float("nan"))
+    g = layers[1]
+    T.paged_attention_decode(alone, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                             q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=256)
+    torch.cuda.synchronize()
+    assert not torch.isnan(outs[1].float()).any()
+    assert torch.equal(outs[1].view(torch.int16), alone.view(torch.int16))
+    with pytest.raises(ValueError):
+        T.paged_attention_decode(alone, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                                 g.softmax_scale, q_len, g.max_context_len, torch.bfloat16, None, g.key_scale,
+                                 g.value_scale, reuse_item_list=True)
+
+
 @pytest.mark.parametrize("case", ["one_partition", "partitions", "shared", "sorted", "queue"])
 def test_empty_sequences_get_zero_rows(cuda, case):
     """A sequence with context length 0 has nothing to attend to: its output rows are zero in every launch mode

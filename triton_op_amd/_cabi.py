@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
 PA_DECODE_ABI_VERSION = 3
 PA_DECODE_WORKSPACE_BYTES = 64
+PA_DECODE_FLAG_REUSE_ITEM_LIST = 1
 PA_DTYPE_BF16, PA_DTYPE_FP8_E4M3FN = 0, 1
 PA_QUANT_NONE, PA_QUANT_PER_TENSOR, PA_QUANT_PER_TOKEN = -1, 0, 1
 
@@ -35,7 +36,7 @@ EXPORTED_SYMBOLS = (
 
 class PaDecodeArgs(C.Structure):
     _fields_ = (
-        [("struct_size", C.c_uint32), ("reserved0", C.c_int32)]
+        [("struct_size", C.c_uint32), ("flags", C.c_int32)]
         + [(n, C.c_void_p) for n in (
             "output", "query", "key_cache", "value_cache", "context_lens", "block_tables", "q_lens",
             "query_scale", "key_scale", "value_scale", "alibi_slopes", "sinks", "exp_sums", "max_logits", "tmp_output",

@@ -20,8 +20,8 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 
 constexpr int kHeadSize = 128;
-// PaDecodeArgs.reserved0 as the kernels see it (the launch layer sets it in its own copy of the arguments)
-constexpr int kFlagSortedItems = 1;  // the workspace holds the planning kernel's item list
+// PaDecodeArgs.flags as the kernels see it (the launch layer sets it in its own copy of the arguments)
+constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning kernel's item list
 // Workspace layout (int32 words): [0], [1] counters of the queued launch, [2] number of listed items,
 // [16 + 2i], [17 + 2i] sequence and partition index of item i.
 constexpr int kPlanHeaderWords = 16;

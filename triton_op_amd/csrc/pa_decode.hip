@@ -43,6 +43,7 @@ int check_common(const PaDecodeArgs* a) {
       a->max_num_partitions <= 0)
     return PA_ERR_BAD_SHAPE;
   if (a->partition_size <= 0 || a->partition_size % 256) return PA_ERR_BAD_SHAPE;
+  if (a->flags & ~PA_DECODE_FLAG_REUSE_ITEM_LIST) return PA_ERR_BAD_SHAPE;
   if (a->workspace ? a->workspace_bytes < PA_DECODE_WORKSPACE_BYTES : a->workspace_bytes != 0) return PA_ERR_BAD_SHAPE;
   if (a->head_size != kHeadSize) return PA_ERR_UNSUPPORTED;
   if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;  // the reference's limit
@@ -112,16 +113,18 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
     long long resident = (long long)device_num_cus() * 4 * OCC / W;
     resident = resident < blocks ? resident : blocks;
     PaDecodeArgs k = a;
-    k.reserved0 = 0;
+    k.flags = 0;
     hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)resident),
                        dim3(64 * W), 0, stream, k);
   } else {
     PaDecodeArgs k = a;
-    k.reserved0 = 0;
+    k.flags = 0;
     if (use_sorted_items(a, blocks, 4 * OCC / W)) {
-      const int rc = launch_plan(a, stream);
-      if (rc) return rc;
-      k.reserved0 = kFlagSortedItems;
+      if (!(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST)) {
+        const int rc = launch_plan(a, stream);
+        if (rc) return rc;
+      }
+      k.flags = kFlagSortedItems;
     }
     hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)blocks), dim3(64 * W), 0,
                        stream, k);
@@ -171,11 +174,13 @@ int launch_partition_shared(const PaDecodeArgs& a, hipStream_t stream) {
   // per CU is worth more than a deeper ring (measured); with them it needs about 140
   constexpr int kWorkgroupsPerCu = PT ? 3 : 4;
   PaDecodeArgs k = a;
-  k.reserved0 = 0;
+  k.flags = 0;
   if (use_sorted_items(a, blocks, kWorkgroupsPerCu)) {
-    const int rc = launch_plan(a, stream);
-    if (rc) return rc;
-    k.reserved0 = kFlagSortedItems;
+    if (!(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST)) {
+      const int rc = launch_plan(a, stream);
+      if (rc) return rc;
+    }
+    k.flags = kFlagSortedItems;
   }
   if constexpr (PT)
     hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, k);

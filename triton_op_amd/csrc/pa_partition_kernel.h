@@ -151,7 +151,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     h = (int)(wid % Hkv);
     rt = (int)((wid / Hkv) % RT);
     const long long item = wid / ((long long)Hkv * RT);
-    if (a.reserved0 & kFlagSortedItems) {
+    if (a.flags & kFlagSortedItems) {
       // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
       if (item >= sload_i32(a.workspace + 2)) return;
       b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);

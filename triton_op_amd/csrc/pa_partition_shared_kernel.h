@@ -49,7 +49,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int h = (int)(wid % Hkv);
   const long long item = wid / Hkv;
   int b, part;
-  if (a.reserved0 & kFlagSortedItems) {
+  if (a.flags & kFlagSortedItems) {
     // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
     if (item >= sload_i32(a.workspace + 2)) return;
     b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);

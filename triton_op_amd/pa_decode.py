@@ -115,6 +115,7 @@ def plan_decode(
     query_lens: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
     sinks: Optional[torch.Tensor] = None,
+    reuse_item_list: bool = False,
 ) -> DecodePlan:
     # ---- shapes (pa_decode_triton_gluon_fp8.py:1703-1722) ------------------------------------
     if output.dim() != 3:
@@ -240,6 +241,8 @@ def plan_decode(
 
     if not output.is_cuda:
         raise ValueError("paged_attention_decode runs on the GPU only (there is no CPU path); got a CPU tensor")
+    if reuse_item_list and workspace is None:
+        raise ValueError("reuse_item_list needs the workspace the earlier call left its item list in")
 
     # ---- partitioning: the launch / tuning layer ---------------------------------------------------------
     max_seq = max(1, int(max_sequence_length))
@@ -314,6 +317,9 @@ def plan_decode(
         raise ValueError(f"workspace must be a contiguous int32 tensor of >= {_cabi.PA_DECODE_WORKSPACE_BYTES} bytes on {dev}")
     a.workspace = workspace.data_ptr()
     a.workspace_bytes = workspace.numel() * 4
+    # the caller's word that `workspace` already holds the item list of a call with the same sequence lengths
+    # and partitioning (the previous layer of this decode step): the planning kernel is skipped
+    a.flags = _cabi.PA_DECODE_FLAG_REUSE_ITEM_LIST if reuse_item_list else 0
     a.num_seqs, a.num_kv_heads, a.group_size, a.q_len = num_seqs, num_kv_heads, group, q_len
     a.head_size, a.block_size = head_size, block_size
     a.max_num_partitions, a.partition_size = max_parts, partition_size
@@ -358,6 +364,7 @@ def paged_attention_decode(
     query_lens: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
     sinks: Optional[torch.Tensor] = None,
+    reuse_item_list: bool = False,
 ) -> Dict[str, object]:
     """Split-KV paged-attention decode; writes `output` in place on torch's current stream and
     returns the partition buffers under the reference's keys."""
@@ -366,7 +373,7 @@ def paged_attention_decode(
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
         num_sequence_partitions, alibi_slopes, exp_sums=exp_sums, max_logits=max_logits,
         tmp_output=tmp_output, partition_size=partition_size, query_lens=query_lens, workspace=workspace,
-        sinks=sinks)
+        sinks=sinks, reuse_item_list=reuse_item_list)
     plan.run()
     return {
         "temporary_output": plan.tmp_output,
