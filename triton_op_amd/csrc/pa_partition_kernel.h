@@ -524,7 +524,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
             p2 *= vs_cur[j][2];
             p3 *= vs_cur[j][3];
           }
-          int hi = 0, lo = 0;
+          // both halves of a packed word are written, so its previous value is irrelevant: a register whose
+          // value is dead (a logit) stands in for it; an explicit zero would cost a move per word
+          int hi = (int)__float_as_uint(s[nt][j][0]), lo = (int)__float_as_uint(s[nt][j][1]);
           hi = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, hi, false);
           hi = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, hi, true);
           const f32x2 b01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
