@@ -96,15 +96,6 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs
   write_token<TO_FP8>(a, t, h, slot, lane);
 }
 
-// ---- append, many tokens (prefill): one workgroup per (16 tokens, up to 4 kv heads) -----------------------------
-// Written token by token the V cache takes 128 separate one-byte stores per token and head (a token is one
-// byte of every head dim's row) and the K cache 2-byte ones; prefill appends runs of tokens to consecutive slots,
-// so here a GROUP, a run of up to 16 tokens that fill consecutive slots of one 16-slot aligned segment of a
-// page, is quantised together: 256 threads load the rows 16 bytes at a time, K leaves as 16-byte (token, chunk)
-// cells, and V is turned through LDS so that each head dim's row gets its 16 tokens in one 16-byte store.
-// A workgroup owns the groups that START among its 16 tokens (a group may reach into the next workgroup's
-// tokens, which then skips them); with more than four groups among its tokens (scattered slots) it writes its
-// tokens one by one like the kernel above.
 // lane exchanges inside a row of 16 lanes on the vector ALU (DPP), not through the LDS crossbar
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
@@ -160,6 +151,15 @@ __device__ __forceinline__ void quantize8(const float (&x)[8], float s, u32x2& o
   }
 }
 
+// ---- append, many tokens (prefill): one workgroup per (16 tokens, up to 4 kv heads) -----------------------------
+// Written token by token the V cache takes 128 separate one-byte stores per token and head (a token is one
+// byte of every head dim's row) and the K cache 2-byte ones; prefill appends runs of tokens to consecutive slots,
+// so here a GROUP, a run of up to 16 tokens that fill consecutive slots of one 16-slot aligned segment of a
+// page, is quantised together: 256 threads load the rows 16 bytes at a time, K leaves as 16-byte (token, chunk)
+// cells, and V is turned through LDS so that each head dim's row gets its 16 tokens in one 16-byte store.
+// A workgroup owns the groups that START among its 16 tokens (a group may reach into the next workgroup's
+// tokens, which then skips them); with more than four groups among its tokens (scattered slots) it writes its
+// tokens one by one like the kernel above.
 constexpr int kHeadsPerWorkgroup = 4;  // kv heads one workgroup of the tile kernel walks, their rows all requested first
 
 // one kv head of a group: kr, vr are this thread's 16 bytes of the token's K and V row
