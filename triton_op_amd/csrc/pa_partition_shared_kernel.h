@@ -73,7 +73,15 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   // while tile 3 rarely is: which wave computes which tile rotates from workgroup to workgroup, so that no
   // SIMD collects the busy tiles of every resident workgroup (worth ~3 % on ragged query lengths).  Which
   // wave fetches which quarter of a step does not rotate.
-  const int row0 = 16 * ((wave + b + h + part) & 3);  // this wave's query tile
+  // With at most two busy tiles (32 query rows) two of the four waves would only fetch, and a busy wave's chain of
+  // 64 tokens' logits, softmax and P per step is what the step waits for.  Then each tile is shared by TWO waves
+  // that take half of every step's tokens each (tiles 0-1 and 2-3 of the step), with (m, l, O) of their own, merged
+  // through LDS at the end: half the chain per wave, all four waves busy (measured on 32 rows: 104 -> 95 us with
+  // per-token scales, 94 -> 85 us without).
+  const int role = (wave + b + h + part) & 3;
+  const bool half_mode = rows_valid <= 32;
+  const int half = half_mode ? role >> 1 : 0;             // which half of every step's tokens this wave takes
+  const int row0 = 16 * (half_mode ? role & 1 : role);    // this wave's query tile
   const bool has_rows = row0 < rows_valid;  // else the wave only helps to fetch
 
   // ---- cache addressing ----------------------------------------------------------------------------------
@@ -235,34 +243,39 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // ---- one step of 64 tokens out of LDS: the arithmetic of pa_partition_kernel's FP8 step, one row tile ----
-  auto compute = [&]<bool FULL>(const StepLds& st, int tok0) {
-    f32x4 s[4];
+  // HALF: this wave takes tiles 2*half, 2*half+1 of the step (32 tokens) instead of all four
+  auto compute = [&]<bool FULL, bool HALF>(const StepLds& st, int tok0) {
+    constexpr int T = HALF ? 2 : 4;       // 16-token tiles of the step this wave works on
+    const int jb = HALF ? 2 * half : 0;   // the first of them
+    f32x4 s[T];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int jj = 0; jj < T; ++jj) {
+      const int j = jb + jj;
       const u32x4 k0 = st.k[j][0][lane], k1 = st.k[j][1][lane];
       const i32x8 ka = {(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
-      s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      s[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi, s[j], 0, 0, 0, 0, 0, 0);
-      s[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[j], 0, 0, 0, 0, 0, 0);
+      s[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+      s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi, s[jj], 0, 0, 0, 0, 0, 0);
+      s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[jj], 0, 0, 0, 0, 0, 0);
     }
     // P is produced already multiplied by pmul = 256 / v_run (per-token V scales: v_run is the running
     // maximum of the scales, P then also carries v_scale / v_run <= 1 and the accumulator is kept in units
     // of v_run): log2(pmul) rides in the exponent's additive term, so it costs nothing per element
     float vfac = 1.f, log2_pmul = 8.f, inv_pmul = 1.f / 256.f;
-    f32x4 ks_cur[PER_TOKEN ? 4 : 1], vs_cur[PER_TOKEN ? 4 : 1];
+    f32x4 ks_cur[PER_TOKEN ? T : 1], vs_cur[PER_TOKEN ? T : 1];
     if constexpr (PER_TOKEN) {
       float vmx = 0.f;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        ks_cur[j] = *reinterpret_cast<const f32x4*>(&st.sc[j][0][4 * kg]);
-        vs_cur[j] = *reinterpret_cast<const f32x4*>(&st.sc[j][1][4 * kg]);
+      for (int jj = 0; jj < T; ++jj) {
+        const int j = jb + jj;
+        ks_cur[jj] = *reinterpret_cast<const f32x4*>(&st.sc[j][0][4 * kg]);
+        vs_cur[jj] = *reinterpret_cast<const f32x4*>(&st.sc[j][1][4 * kg]);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           if constexpr (!FULL) {
             const int col = tok0 + 16 * j + 4 * kg + r;
-            vs_cur[j][r] = col < ctx ? vs_cur[j][r] : 0.f;
+            vs_cur[jj][r] = col < ctx ? vs_cur[jj][r] : 0.f;
           }
-          vmx = fmaxf(vmx, vs_cur[j][r]);
+          vmx = fmaxf(vmx, vs_cur[jj][r]);
         }
       }
       vmx = quad_row_max(vmx);
@@ -275,17 +288,17 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     // FULL: the row's scale (>= 0 on this path) is applied inside the exponent's fma, and to the maximum once
     float mx = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int jj = 0; jj < T; ++jj) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float v = s[j][r];
-        if constexpr (PER_TOKEN) v *= ks_cur[j][r];
+        float v = s[jj][r];
+        if constexpr (PER_TOKEN) v *= ks_cur[jj][r];
         if constexpr (!FULL) {
-          const int col = tok0 + 16 * j + 4 * kg + r;
+          const int col = tok0 + 16 * (jb + jj) + 4 * kg + r;
           v = v * rscale + slope2 * (float)(col - ctx + 1);
           v = col < limit ? v : -INFINITY;
         }
-        s[j][r] = v;
+        s[jj][r] = v;
         mx = fmaxf(mx, v);
       }
     }
@@ -298,9 +311,9 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     const float e_add = log2_pmul - m_safe;
     const float e_mul = FULL ? rscale : 1.f;
     float psum = 0.f;
-    uint32_t ph[4], pl[4];
+    uint32_t ph[4] = {0u, 0u, 0u, 0u}, pl[4] = {0u, 0u, 0u, 0u};  // (HALF: the tiles that are not this wave's hold P = 0)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < T; ++j) {
       float p0 = fast_exp2(__builtin_fmaf(s[j][0], e_mul, e_add));
       float p1 = fast_exp2(__builtin_fmaf(s[j][1], e_mul, e_add));
       float p2 = fast_exp2(__builtin_fmaf(s[j][2], e_mul, e_add));
@@ -340,15 +353,18 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     // over (tile kg's 16 tokens with P head, the same 16 tokens with P residual), so the A operand is the V
     // bytes twice -- read from LDS twice, which costs no VALU slot
     const i32x8 pb = {(int)ph[0], (int)ph[1], (int)ph[2], (int)ph[3], (int)pl[0], (int)pl[1], (int)pl[2], (int)pl[3]};
+    // after the transpose lane group kg holds P of the step's tile kg, or, HALF, of this wave's tile kg (kg < 2)
+    // and zeros (kg >= 2), which meet this wave's tiles' V bytes once more
+    const int vj = HALF ? jb + (kg & 1) : kg;
     int nvalid = 16;
     if constexpr (!FULL) {
       // V bytes of tokens at or beyond ctx are zeroed (stale cache contents may decode to NaN)
-      nvalid = ctx - (tok0 + 16 * kg);
+      nvalid = ctx - (tok0 + 16 * vj);
       nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
     }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const u32x4* vp = &st.v[kg][16 * db + li];
+      const u32x4* vp = &st.v[vj][16 * db + li];
       typedef const volatile __attribute__((address_space(3))) u32x4* LdsVec;
       u32x4 v0 = *vp;
       u32x4 v1 = *(LdsVec)vp;  // a second LDS read, not a register copy
@@ -397,15 +413,28 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   // in different loops: all of them pass the same number of barriers.
   if (has_rows) {
     const int n_fast = rs_nonneg ? (n_full < n_steps ? n_full : n_steps) : 0;
-    while (s < n_fast) {
-      enter_step();
-      compute.template operator()<true>(stage[slot], tok0);
-      leave_step();
-    }
-    while (s < n_steps) {
-      enter_step();
-      compute.template operator()<false>(stage[slot], tok0);
-      leave_step();
+    if (half_mode) {
+      while (s < n_fast) {
+        enter_step();
+        compute.template operator()<true, true>(stage[slot], tok0);
+        leave_step();
+      }
+      while (s < n_steps) {
+        enter_step();
+        compute.template operator()<false, true>(stage[slot], tok0);
+        leave_step();
+      }
+    } else {
+      while (s < n_fast) {
+        enter_step();
+        compute.template operator()<true, false>(stage[slot], tok0);
+        leave_step();
+      }
+      while (s < n_steps) {
+        enter_step();
+        compute.template operator()<false, false>(stage[slot], tok0);
+        leave_step();
+      }
     }
   } else {
     while (s < n_steps) {
@@ -415,10 +444,9 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   }
   __syncthreads();  // the stage buffers are free
 
-  // ---- epilogue: every wave writes its own row tile -----------------------------------------------------------
-  if (!has_rows) {
-    // a tile of padding rows only (a ragged batch): the rows read as "no visible key"
-    for (int r = row0 + kg; r < row0 + 16 && r < Ge; r += 4) {
+  // a tile of padding rows only (a ragged batch): the rows read as "no visible key"
+  auto write_padding_rows = [&](int first_row) {
+    for (int r = first_row + kg; r < first_row + 16 && r < Ge; r += 4) {
       if (li == 0) {
         a.max_logits[es_off + r] = -INFINITY;
         a.exp_sums[es_off + r] = 0.f;
@@ -426,6 +454,54 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
       *reinterpret_cast<u32x4*>(tmp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
       if (direct) *reinterpret_cast<u32x4*>(outp + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
     }
+  };
+
+  // ---- two waves per tile: the second hands its (m, l, O) to the first ------------------------------------------
+  float acc_unit = (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f);
+  if (half_mode) {
+    // per tile: m and l of the 16 rows (lanes 0..15) and the 32 accumulator registers of all 64 lanes, in units of 1
+    constexpr int kMergeFloats = 2 * 16 + 32 * 64;
+    static_assert(sizeof(StepLds) * NB >= 2 * kMergeFloats * 4 + 2 * 16 * kORowBytes, "room for the merge buffers");
+    float* mb = reinterpret_cast<float*>(&stage[0]) + (row0 >> 4) * kMergeFloats;
+    if (has_rows && half == 1) {
+      const float lt = quad_row_sum(l_run);
+      if (kg == 0) {
+        mb[li] = m_run;
+        mb[16 + li] = lt;
+      }
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mb[32 + (4 * db + r) * 64 + lane] = acc[db][r] * acc_unit;
+      }
+    }
+    __syncthreads();
+    if (half == 1) {
+      // done with its tile; the tiles 2 and 3 of a larger group hold padding rows only, which these two waves write
+      write_padding_rows(32 + row0);
+      return;
+    }
+    if (has_rows) {
+      const float m1 = mb[li], l1 = mb[16 + li];
+      const float l0 = quad_row_sum(l_run);
+      const float mm = fmaxf(m_run, m1);
+      const float m_safe = mm == -INFINITY ? 0.f : mm;
+      const float w0 = fast_exp2(m_run - m_safe), w1 = fast_exp2(m1 - m_safe);  // exp2(-inf) = 0: a half that saw no key
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[db][r] = acc[db][r] * (acc_unit * w0) + mb[32 + (4 * db + r) * 64 + lane] * w1;
+      }
+      m_run = mm;
+      // l_run becomes this lane's share of the merged sum: the row total in lane group 0, nothing elsewhere
+      l_run = kg == 0 ? l0 * w0 + l1 * w1 : 0.f;
+      acc_unit = 1.f;
+    }
+  }
+
+  // ---- epilogue: every wave writes its own row tile -----------------------------------------------------------
+  if (!has_rows) {
+    write_padding_rows(row0);
     return;
   }
   float l_tot = quad_row_sum(l_run);
@@ -433,13 +509,14 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     l_tot = 0.f;
     m_run = -INFINITY;
   }
-  const float acc_unit = (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f);
   const float inv = l_tot > 0.f ? v_tensor_scale * acc_unit / l_tot : 0.f;
   if (row < Ge && kg == 0) {
     a.max_logits[es_off + row] = m_run * (1.0f / kLog2e);
     a.exp_sums[es_off + row] = l_tot;
   }
-  char* olds = reinterpret_cast<char*>(&stage[0]) + wave * (16 * kORowBytes);
+  // wave-private staging for the transposed store (two waves per tile: behind the merge buffers, one per tile)
+  char* olds = reinterpret_cast<char*>(&stage[0]) +
+               (half_mode ? 2 * (2 * 16 + 32 * 64) * 4 + (row0 >> 4) * (16 * kORowBytes) : wave * (16 * kORowBytes));
   store_partial_tile(olds, acc, inv, tmp + (int64_t)row0 * a.stride_tmp_g * 2, a.stride_tmp_g * 2,
                      direct ? outp + (int64_t)row0 * a.stride_out_h * 2 : nullptr, a.stride_out_h * 2, Ge - row0, lane);
 }
