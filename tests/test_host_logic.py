@@ -78,6 +78,9 @@ def test_partition_size_choices():
     assert f(128, 8, 16, 32768, 1024, 256) == 8192  # c3
     assert f(256, 8, 64, 65536, 16, 256) == 8192   # c5: 64 rows = 4 row tiles sharing one workgroup's page stream
     assert f(4, 8, 32, 131072, 16, 256) == 5632    # few long sequences, 2 row tiles: 24 partitions fill the GPU
+    assert f(32, 4, 32, 4096, 16, 256) == 1024     # short partitions: two workgroups per CU (36.6 us against 39.4 for 768)
+    assert f(4, 8, 64, 16384, 16, 256) == 1024     # measured 43.0 us against 47.6 us for 768
+    assert f(64, 4, 32, 4096, 16, 256) == 1536     # measured 59.9 us against 61.9 (2048) and 64.9 (1024)
     assert f(4, 1, 8, 1024, 16, 256) == 1024       # c1: tiny; one partition, no second kernel
     assert f(48, 8, 8, 4096, 16, 256) == 4096      # three quarters of the wave slots filled: still one partition
     assert f(4, 8, 8, 4096, 16, 256) == 512        # 32 rows only: eight partitions each
