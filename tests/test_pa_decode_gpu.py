@@ -128,6 +128,13 @@ CASES = {
     "fp8_token_transV_bs64_g8_q3": dict(batch=2, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(1500, 200),
                                         block_size=64, transposed_v=True, q_len=3, scale_mode="token"),
     "fp8_g8_q4_long": dict(batch=2, num_q_heads=8, num_kv_heads=1, context_lens=_ctx(9000, 4097), q_len=4),
+    # at most two busy tiles of a four-tile group: two waves share a tile and split each step's tokens; contexts
+    # so short that the second wave sees no key at all, and the padding tiles are written by the waves left over
+    "fp8_ragged_two_waves_per_tile": dict(batch=5, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(5, 33, 700, 31, 257),
+                                          q_len=4, q_lens=_ctx(1, 2, 1, 2, 2)),
+    "fp8_token_ragged_two_waves_per_tile": dict(batch=5, num_q_heads=32, num_kv_heads=2,
+                                                context_lens=_ctx(17, 64, 1000, 2, 300), q_len=4,
+                                                q_lens=_ctx(2, 1, 2, 2, 1), scale_mode="token"),
     "bf16_transV_bs64": dict(batch=2, num_q_heads=8, num_kv_heads=2, context_lens=_ctx(150, 300), block_size=64,
                              kv_dtype="bf16", scale_mode="none", transposed_v=True),
 }
