@@ -53,6 +53,22 @@ def build(verbose: bool = True, extra_flags=()) -> str:
     return LIB_PATH
 
 
+NATIVE_SMOKE_SRC = os.path.join(HERE, "..", "tests", "native", "abi_smoke.cpp")
+NATIVE_SMOKE_BIN = os.path.join(HERE, "..", "tests", "native", "abi_smoke")
+
+
+def build_native_smoke(verbose: bool = True) -> str:
+    """The C++ caller of the C ABI that the GPU tests run (tests/native/abi_smoke.cpp): no Python, no torch."""
+    cmd = [find_hipcc(), "-O2", NATIVE_SMOKE_SRC, "-I" + os.path.join(HERE, "..", "include"), "-L" + HERE,
+           "-lpa_decode", "-Wl,-rpath,$ORIGIN/../../triton_op_amd", "-o", NATIVE_SMOKE_BIN]
+    if verbose:
+        print("[triton_op_amd.build]", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
+    return NATIVE_SMOKE_BIN
+
+
 def is_stale() -> bool:
     if not os.path.exists(LIB_PATH):
         return True
@@ -62,3 +78,4 @@ def is_stale() -> bool:
 
 if __name__ == "__main__":
     build()
+    build_native_smoke()
