@@ -25,13 +25,15 @@ extern "C" {
 /* Smallest useful size of the optional device workspace.  Its first 64 bytes hold a work-item counter: with
  * it, batches with per-sequence query lengths are launched as a resident grid that pulls live (sequence,
  * partition, row tile, head) items from the counter instead of one workgroup per possible item.  These 64
- * bytes must be zero before the first call; every call leaves them zero.  A workspace of
+ * bytes must be zero before the first call; every call leaves the counters (the first 8 bytes) zero, the rest of
+ * the 64 bytes is scratch that a call writes before it reads it.  A workspace of
  * pa_decode_workspace_bytes() bytes also has room for the work-item list of the sorted dispatch: in launches of
  * several rounds of workgroups a small planning kernel lists the live (sequence, partition) items, whole
  * partitions first and the sequences' last, partial partitions by decreasing length, and the partition kernel
- * takes its items from the list (longest-first keeps the end of a ragged batch's launch busy).  The list is
- * rewritten by every call (unless PA_DECODE_FLAG_REUSE_ITEM_LIST says it is still good).  Calls that may overlap
- * on the GPU need a workspace each. */
+ * takes its items from the list (longest-first keeps the end of a ragged batch's launch busy); it also lists the
+ * sequences that have more than one partition, which are all that pa_decode's reduce stage then visits.  The
+ * lists are rewritten by every call (unless PA_DECODE_FLAG_REUSE_ITEM_LIST says they are still good).  Calls that
+ * may overlap on the GPU need a workspace each. */
 #define PA_DECODE_WORKSPACE_BYTES 64
 /*
  * flags: the workspace still holds the item list that an earlier call built for the SAME context_lens contents,
@@ -132,7 +134,8 @@ uint32_t pa_decode_args_size(void);
 const char* pa_decode_error_string(int code);
 /* hipError_t of the last failed launch on the calling thread (0 if none). */
 int pa_decode_last_hip_error(void);
-/* Workspace size that enables every launch mode for a batch of this shape (see PA_DECODE_WORKSPACE_BYTES). */
+/* Workspace size that enables every launch mode for a batch of this shape (see PA_DECODE_WORKSPACE_BYTES):
+ * 64 + 8 * num_seqs * max_num_partitions + 4 * num_seqs. */
 int64_t pa_decode_workspace_bytes(int32_t num_seqs, int32_t max_num_partitions);
 
 /*

@@ -52,9 +52,9 @@ def test_struct_layout_and_version(pa_lib):
 
 
 def test_workspace_size_rule(pa_lib):
-    # 64 bytes of counters + one (sequence, partition) pair of int32 per possible item
-    assert pa_lib.pa_decode_workspace_bytes(256, 8) == 64 + 8 * 256 * 8
-    assert pa_lib.pa_decode_workspace_bytes(1, 1) == 72
+    # 64 bytes of counters + one (sequence, partition) pair of int32 per possible item + one int32 per sequence
+    assert pa_lib.pa_decode_workspace_bytes(256, 8) == 64 + 8 * 256 * 8 + 4 * 256
+    assert pa_lib.pa_decode_workspace_bytes(1, 1) == 76
     assert pa_lib.pa_decode_workspace_bytes(0, 4) == _cabi.PA_DECODE_WORKSPACE_BYTES
 
 

@@ -348,7 +348,10 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, scale_mode=scale_mode)
     g = wl.to(cuda)
     outs = []
-    for ws_bytes in (None, 64):  # None: the entry point sizes the workspace for the item list; 64: counters only
+    parts = -(-int(ctx.max()) // 256)
+    # None: the entry point sizes the workspace for both lists (sorted dispatch, listed reduce); room for the item
+    # list only (sorted dispatch, reduce over every sequence); 64: counters only (grid order)
+    for ws_bytes in (None, 64 + 8 * batch * parts, 64):
         ws = None if ws_bytes is None else torch.zeros(ws_bytes // 4, dtype=torch.int32, device=cuda)
         out = torch.full_like(g.query, float("nan"))
         plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
@@ -360,6 +363,7 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
         torch.cuda.synchronize()
         outs.append(out.cpu())
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 

@@ -25,6 +25,9 @@ constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning k
 // Workspace layout (int32 words): [0], [1] counters of the queued launch, [2] number of listed items,
 // [16 + 2i], [17 + 2i] sequence and partition index of item i.
 constexpr int kPlanHeaderWords = 16;
+// word of the workspace header: how many sequences have more than one partition (their numbers are the last
+// num_seqs words of a workspace that is long enough for them)
+constexpr int kPlanMultiWord = 5;
 constexpr int kStepTokens = 64;     // tokens per pipeline step (4 tiles of 16)
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kPRowBytes = 144;     // 64 tokens * 2 B + 16 B pad per query row of the P tile

@@ -34,6 +34,8 @@ __global__ void pa_fp8_decode_kernel(const uint8_t* codes, float* out, int n) {
 }
 
 thread_local int g_last_hip_error = 0;
+// set by the partition stage's launch: did it go through the planning kernel's lists (sorted dispatch)?
+thread_local bool g_used_item_lists = false;
 
 int check_common(const PaDecodeArgs* a) {
   if (!a) return PA_ERR_NULL_POINTER;
@@ -77,6 +79,10 @@ bool use_queue(const PaDecodeArgs& a) {
 // Bytes of workspace the sorted dispatch needs: the header and one (sequence, partition) pair per possible item.
 long long plan_workspace_bytes(int num_seqs, int max_num_partitions) {
   return 4LL * kPlanHeaderWords + 8LL * num_seqs * max_num_partitions;
+}
+// ... and one more word per sequence for the list of the sequences with more than one partition
+long long full_workspace_bytes(int num_seqs, int max_num_partitions) {
+  return plan_workspace_bytes(num_seqs, max_num_partitions) + 4LL * num_seqs;
 }
 
 // The sorted dispatch pays a small extra kernel, and ordering only matters when workgroups are handed out in
@@ -125,6 +131,7 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
         if (rc) return rc;
       }
       k.flags = kFlagSortedItems;
+      g_used_item_lists = true;
     }
     hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)blocks), dim3(64 * W), 0,
                        stream, k);
@@ -181,6 +188,7 @@ int launch_partition_shared(const PaDecodeArgs& a, hipStream_t stream) {
       if (rc) return rc;
     }
     k.flags = kFlagSortedItems;
+    g_used_item_lists = true;
   }
   if constexpr (PT)
     hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, k);
@@ -233,6 +241,25 @@ int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
   return PA_OK;
 }
 
+// The reduce stage of a call whose partition stage went through the planning kernel: only the sequences with
+// more than one partition are visited, by a grid of at most eight workgroups per CU that walks their units.
+int launch_reduce_listed(const PaDecodeArgs* a, void* hip_stream) {
+  const long long units = (long long)a->num_seqs * a->num_kv_heads * ((a->q_len * a->group_size + 15) / 16);
+  const long long cap = 8LL * device_num_cus();
+  const unsigned blocks = (unsigned)(units < cap ? units : cap);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  if (units * 16 >= 16384)
+    hipLaunchKernelGGL((pa_reduce_listed_kernel<4>), dim3(blocks), dim3(256), 0, stream, *a);
+  else
+    hipLaunchKernelGGL((pa_reduce_listed_kernel<1>), dim3(blocks), dim3(1024), 0, stream, *a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return PA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -243,7 +270,7 @@ int pa_decode_last_hip_error(void) { return g_last_hip_error; }
 
 int64_t pa_decode_workspace_bytes(int32_t num_seqs, int32_t max_num_partitions) {
   if (num_seqs <= 0 || max_num_partitions <= 0) return PA_DECODE_WORKSPACE_BYTES;
-  return plan_workspace_bytes(num_seqs, max_num_partitions);
+  return full_workspace_bytes(num_seqs, max_num_partitions);
 }
 
 const char* pa_decode_error_string(int code) {
@@ -382,10 +409,18 @@ int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) { return launch_re
 
 int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
   if (a && a->struct_size == sizeof(PaDecodeArgs) && !a->output) return PA_ERR_NULL_POINTER;
+  g_used_item_lists = false;
   int rc = pa_decode_partition(a, hip_stream);
   if (rc) return rc;
   // the partition kernel has written the rows of every sequence that fits in one partition itself
   if (a->max_num_partitions == 1 && !a->sinks) return PA_OK;
+  if (g_used_item_lists && !a->sinks && a->workspace_bytes >= full_workspace_bytes(a->num_seqs, a->max_num_partitions)) {
+    // (the stride checks of the reduce stage)
+    if (a->stride_out_h % 2 || a->stride_out_s % 2 || a->stride_tmp_g % 2 || a->stride_tmp_p % 2 || a->stride_tmp_h % 2 ||
+        a->stride_tmp_s % 2)
+      return PA_ERR_BAD_SHAPE;
+    return launch_reduce_listed(a, hip_stream);
+  }
   return launch_reduce(a, hip_stream, true);
 }
 

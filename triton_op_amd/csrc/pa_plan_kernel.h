@@ -21,6 +21,7 @@ __global__ __launch_bounds__(1024) void pa_plan_kernel(const PaDecodeArgs a) {
   __shared__ int s_wave[16];
   __shared__ int s_hist[kPlanClasses];
   __shared__ int s_base[kPlanClasses];
+  __shared__ int s_multi;  // sequences with more than one partition
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int B = a.num_seqs, ps = a.partition_size, P = a.max_num_partitions;
   const int per = (B + 1023) / 1024;  // sequences per thread (contiguous), at most 4
@@ -53,7 +54,18 @@ __global__ __launch_bounds__(1024) void pa_plan_kernel(const PaDecodeArgs a) {
   }
   if (lane == 63) s_wave[wave] = incl;
   if (tid < kPlanClasses) s_hist[tid] = 0;
+  if (tid == 0) s_multi = 0;
   __syncthreads();
+  // the sequences the reduce kernel has work for, in any order, at the end of a workspace that has room for them
+  const bool has_multi_list = a.workspace_bytes >= 4LL * kPlanHeaderWords + 8LL * B * P + 4LL * B;
+  if (has_multi_list) {
+    int* multi = a.workspace + (a.workspace_bytes / 4 - B);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int b = tid * per + i;
+      if (i < per && b < B && nfull[i] + (tail[i] > 0 ? 1 : 0) > 1) multi[atomicAdd(&s_multi, 1)] = b;
+    }
+  }
   int wave_off = 0, total_full = 0;
 #pragma unroll
   for (int w = 0; w < 16; ++w) {
@@ -90,6 +102,7 @@ __global__ __launch_bounds__(1024) void pa_plan_kernel(const PaDecodeArgs a) {
       s_hist[c] = 0;  // becomes the class's cursor
     }
     a.workspace[2] = total_full + acc;
+    a.workspace[kPlanMultiWord] = has_multi_list ? s_multi : -1;
   }
   __syncthreads();
   int* items = a.workspace + kPlanHeaderWords;

@@ -135,16 +135,10 @@ __device__ __forceinline__ void reduce_four_rows(const PaDecodeArgs& a, int b, i
   }
 }
 
+// one unit of the reduce: 16 output rows (row tile rt) of kv head h of sequence b, by one workgroup
 template <bool SKIP_SINGLE, int ROWS>
-__global__ __launch_bounds__(1024 / ROWS) void pa_reduce_kernel(const PaDecodeArgs a) {
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+__device__ __forceinline__ void reduce_unit(const PaDecodeArgs& a, int b, int h, int rt, int lane, int wave) {
   const int Ge = a.q_len * a.group_size;
-  const int RT = (Ge + 15) / 16;
-  const long long wid = blockIdx.x;
-  const int rt = (int)(wid % RT);
-  const int h = (int)((wid / RT) % a.num_kv_heads);
-  const int b = (int)(wid / ((long long)RT * a.num_kv_heads));
   const int row0 = 16 * rt + wave;  // ROWS = 4: this wave's rows are row0 + 4 * rr
   if (row0 >= Ge) return;
 
@@ -166,6 +160,37 @@ __global__ __launch_bounds__(1024 / ROWS) void pa_reduce_kernel(const PaDecodeAr
     if (row >= Ge) break;
     const uint32_t v = row < rows_valid ? reduce_row(a, b, h, row, n, lane) : 0u;
     *reinterpret_cast<uint32_t*>(outp + (int64_t)row * a.stride_out_h * 2) = v;
+  }
+}
+
+template <bool SKIP_SINGLE, int ROWS>
+__global__ __launch_bounds__(1024 / ROWS) void pa_reduce_kernel(const PaDecodeArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int RT = (a.q_len * a.group_size + 15) / 16;
+  const long long wid = blockIdx.x;
+  const int rt = (int)(wid % RT);
+  const int h = (int)((wid / RT) % a.num_kv_heads);
+  const int b = (int)(wid / ((long long)RT * a.num_kv_heads));
+  reduce_unit<SKIP_SINGLE, ROWS>(a, b, h, rt, lane, wave);
+}
+
+// The same over the planning kernel's list of the sequences that have more than one partition (the others got
+// their output rows from the partition kernel): a launch of a few hundred workgroups that walk the list's units,
+// instead of one workgroup per (sequence, head, row tile) of which most would only find out that they have
+// nothing to do (8192 of them cost 9 us on a ragged batch of 256 sequences).
+template <int ROWS>
+__global__ __launch_bounds__(1024 / ROWS) void pa_reduce_listed_kernel(const PaDecodeArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int RT = (a.q_len * a.group_size + 15) / 16;
+  const int per_seq = RT * a.num_kv_heads;
+  const int* list = a.workspace + (a.workspace_bytes / 4 - a.num_seqs);
+  const long long units = (long long)sload_i32(a.workspace + kPlanMultiWord) * per_seq;
+  for (long long u = blockIdx.x; u < units; u += gridDim.x) {
+    const int b = sload_i32(list + u / per_seq);
+    const int r = (int)(u % per_seq);
+    reduce_unit<false, ROWS>(a, b, r / RT, r % RT, lane, wave);
   }
 }
 
