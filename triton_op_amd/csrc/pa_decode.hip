@@ -154,12 +154,27 @@ int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
 // measured and lose: a wave's chain of 1.4 us steps is what a small batch waits for, and more partitions
 // shorten it where more waves per workgroup cannot go below the second kernel's cost anyway.
 int waves_for_partition_size(int partition_size) { return partition_size >= 512 ? 4 : 2; }
+// ... and no more waves than it takes to fill the GPU's wave slots (8 per CU): with 8 workgroups or more per CU
+// one wave each is best (no merge, more independent streams: 256 sequences x 8 kv heads x 512 tokens 57.7 -> 44.8
+// us), with 4 per CU two.  But a wave keeps at most 16 steps (1024 tokens) to itself, or the longest items of a
+// ragged batch finish the launch alone, one slow wave each (256 sequences of 1..4096 tokens: 196 us with one
+// wave per workgroup against 179 us with four).
 int waves_per_workgroup(const PaDecodeArgs& a) {
   static const int forced = [] {
     const char* e = getenv("PA_DECODE_WAVES");
     return e ? atoi(e) : 0;
   }();
-  const int w = forced > 0 ? forced : waves_for_partition_size(a.partition_size);
+  int w = waves_for_partition_size(a.partition_size);
+  if (forced > 0) {
+    w = forced;
+  } else {
+    const long long workgroups = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions *
+                                 ((a.q_len * a.group_size + 15) / 16);
+    const long long slots = 8LL * device_num_cus();
+    int need = 1;  // waves per workgroup that fill the slots, or keep a wave's share at 1024 tokens
+    while (need < w && (workgroups * need < slots || a.partition_size > 1024 * need)) need *= 2;
+    w = need;
+  }
   return w >= 4 ? 4 : (w >= 2 ? 2 : 1);
 }
 
