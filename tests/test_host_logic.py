@@ -232,3 +232,24 @@ def test_header_is_plain_c_and_links(tmp_path):
     res = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
     assert res.returncode == 0, (res.returncode, res.stdout, res.stderr)
     assert "stride" in res.stdout or "size" in res.stdout
+
+
+def test_short_division_of_the_cache_writers_is_the_rounded_quotient(tmp_path):
+    """The KV-cache write kernels divide by a row's scale with a reciprocal and ONE correction of the quotient
+    (pa_kv_cache.hip: quantize8, bf16_amax_to_scale) and must still produce the correctly rounded x / scale of
+    the torch formula (kv_layout.pertoken_quant).  tests/native/short_division_check.c runs the same arithmetic
+    on the host against the compiler's division: exhaustively for per-token scales, widely for arbitrary ones."""
+    import os
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = tmp_path / "short_division_check"
+    subprocess.run([gcc, "-O2", "-ffp-contract=off", os.path.join(root, "tests", "native", "short_division_check.c"),
+                    "-lm", "-o", str(exe)], check=True)
+    res = subprocess.run([str(exe), "8000"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert " 0 mismatches; arbitrary" in res.stdout and res.stdout.rstrip().endswith("amax/448 0 mismatches")

@@ -207,3 +207,36 @@ def test_cache_write_of_many_tokens_matches_the_host_quantiser(cuda, mode, bs, t
         assert torch.equal(ks.cpu()[w], ksr[w]) and torch.equal(vs.cpu()[w], vsr[w])
         assert bool((ks.cpu()[~w] == 7.0).all()) and bool((vs.cpu()[~w] == 7.0).all())
         assert float(ks[int(slots[7]) // bs, 1, int(slots[7]) % bs, 0]) == 1.0
+
+
+@pytest.mark.parametrize("scale_bits", [0x3C7FFFFF, 0x3C800001, 0x3D7FFF80, 0x3DABCDEF, 0x2A800000, 0x55123456],
+                         ids=["all_ones", "one_ulp_over_pow2", "high_significand", "generic", "tiny", "huge"])
+def test_cache_write_with_awkward_per_tensor_scales(cuda, scale_bits):
+    """A caller's per-tensor scale can be any float: the short division of the many-token kernel (one reciprocal,
+    one quotient correction; full division for a significand of all ones or a scale outside 2^-40 .. 2^40) must
+    give the bytes of the torch formula for rows full of powers of two, near-ties and ordinary values."""
+    import triton_op_amd as T
+
+    bs, h, d, toks = 16, 2, 128, 2048
+    g = torch.Generator().manual_seed(scale_bits & 0xffff)
+    scale = torch.tensor([scale_bits], dtype=torch.int32).view(torch.float32)[0]
+    key = (torch.randn(toks, h, d, generator=g) * scale * 100).to(torch.bfloat16)
+    value = (torch.randn(toks, h, d, generator=g) * scale * 100).to(torch.bfloat16)
+    # powers of two and every fp8 midpoint times the scale (rounded to bf16): where a quotient one ulp off shows
+    pw = torch.pow(2.0, torch.arange(-10, 10, dtype=torch.float32))
+    key[0, 0, :20] = (pw * scale).to(torch.bfloat16)
+    grid = torch.arange(0, 256, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    grid = grid[torch.isfinite(grid) & (grid > 0)].sort().values
+    mids = ((grid[1:] + grid[:-1]) / 2)[:d]
+    value[1, 1, : mids.numel()] = (mids * scale).to(torch.bfloat16)
+    slots = torch.randperm(toks // bs, generator=g).repeat_interleave(bs) * bs + torch.arange(toks) % bs
+    kref = L.tokens_to_key_cache((key.float() / scale).clamp(-448, 448).to(torch.float8_e4m3fn).view(toks // bs, bs, h, d))
+    vref = L.tokens_to_value_cache((value.float() / scale).clamp(-448, 448).to(torch.float8_e4m3fn).view(toks // bs, bs, h, d))
+    order = (slots.view(-1, bs)[:, 0] // bs)
+    kc = torch.zeros(kref.shape, dtype=torch.uint8, device=cuda).view(torch.float8_e4m3fn)
+    vc = torch.zeros(vref.shape, dtype=torch.uint8, device=cuda).view(torch.float8_e4m3fn)
+    s_dev = scale.to(cuda)
+    T.kv_cache_write(key.to(cuda), value.to(cuda), kc, vc, slots.to(cuda), s_dev, s_dev)
+    torch.cuda.synchronize()
+    assert torch.equal(kc.cpu().view(torch.uint8)[order], kref.view(torch.uint8))
+    assert torch.equal(vc.cpu().view(torch.uint8)[order], vref.view(torch.uint8))

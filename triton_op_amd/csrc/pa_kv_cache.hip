@@ -114,27 +114,40 @@ __device__ __forceinline__ float row16_max(float v) {
   return v;
 }
 
+// amax / 448 for a row maximum that is a bf16 value: the correctly rounded float32 quotient from the constant
+// reciprocal and one correction of the quotient (the residual amax - 448 q is exact in one fma); checked on the
+// host against the division for every positive bf16 value, subnormal ones included.
+__device__ __forceinline__ float bf16_amax_to_scale(float amax) {
+  constexpr float r = 1.f / kFp8Max;
+  if (__builtin_expect(!(amax < 0x1p127f), 0)) return __fdiv_rn(amax, kFp8Max);  // infinity stays infinity
+  const float q0 = amax * r;
+  return __builtin_fmaf(__builtin_fmaf(-kFp8Max, q0, amax), r, q0);
+}
+
 // Eight values of one row divided by the row's scale and rounded to e4m3fn, four bytes per word.
 // x / s must be the correctly rounded float32 quotient (what the host-side formula computes).  A float division
-// expands to a reciprocal, one correction of it and two corrections of the quotient; with one divisor for the
-// whole row the reciprocal part is done once and a value costs five instructions instead of ten.  That short
-// form is exact while nothing over- or underflows on the way: it is used for scales within 2^-40 .. 2^40 and
-// values below 2^80 (a quotient too small for its residual to be exact is far below the smallest FP8 value and
-// rounds to zero either way); anything else takes the full division.
-__device__ __forceinline__ void quantize8(const float (&x)[8], float s, u32x2& out) {
+// expands to a reciprocal, one correction of it and two corrections of the quotient.  With one divisor for the
+// whole row the reciprocal part is done once, and for a bf16 x one correction of the quotient is enough: the
+// once corrected reciprocal is within an ulp of 1/s, so q0 = x r is within an ulp of x/s, the residual x - s q0
+// is exact in one fma and q0 + residual r rounds to the quotient (on the host: every bf16 x against every
+// scale a bf16 row maximum can give, and 3e5 arbitrary scales, with a first reciprocal 1 ulp off either way;
+// only scales whose significand is all ones can miss) -- three instructions per value instead of ten.
+// That short form needs nothing to over- or underflow on the way: it is used for scales within 2^-40 .. 2^40 and
+// values below 2^80 (`xbound` is any bound of |x|; a quotient too small for its residual to be exact is far
+// below the smallest FP8 value and rounds to zero either way); anything else takes the full division.
+// CLAMP = false: the caller knows |x / s| <= 448 (1 + 2^-23), which converts to +-448 as it is (per-token scales:
+// s = amax / 448 of a row that holds x).
+template <bool CLAMP>
+__device__ __forceinline__ void quantize8(const float (&x)[8], float s, float xbound, u32x2& out) {
   float q[8];
-  float xmax = 0.f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) xmax = fmaxf(xmax, fabsf(x[e]));
   const float as = fabsf(s);
-  if (as > 0x1p-40f && as < 0x1p40f && xmax < 0x1p80f) {
+  if (as > 0x1p-40f && as < 0x1p40f && xbound < 0x1p80f && (__float_as_uint(s) & 0x7fffffu) != 0x7fffffu) {
     const float r0 = __builtin_amdgcn_rcpf(s);
     const float r = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.f), r0, r0);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float q0 = x[e] * r;
-      const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, x[e]), r, q0);
-      q[e] = __builtin_fmaf(__builtin_fmaf(-s, q1, x[e]), r, q1);
+      q[e] = __builtin_fmaf(__builtin_fmaf(-s, q0, x[e]), r, q0);
     }
   } else {
 #pragma unroll
@@ -143,8 +156,13 @@ __device__ __forceinline__ void quantize8(const float (&x)[8], float s, u32x2& o
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
     // clamp like fminf(fmaxf(x, -448), 448) (a NaN becomes -448), then two conversions of two values each
-    const float c0 = __builtin_amdgcn_fmed3f(q[4 * w], -kFp8Max, kFp8Max), c1 = __builtin_amdgcn_fmed3f(q[4 * w + 1], -kFp8Max, kFp8Max);
-    const float c2 = __builtin_amdgcn_fmed3f(q[4 * w + 2], -kFp8Max, kFp8Max), c3 = __builtin_amdgcn_fmed3f(q[4 * w + 3], -kFp8Max, kFp8Max);
+    float c0 = q[4 * w], c1 = q[4 * w + 1], c2 = q[4 * w + 2], c3 = q[4 * w + 3];
+    if constexpr (CLAMP) {
+      c0 = __builtin_amdgcn_fmed3f(c0, -kFp8Max, kFp8Max);
+      c1 = __builtin_amdgcn_fmed3f(c1, -kFp8Max, kFp8Max);
+      c2 = __builtin_amdgcn_fmed3f(c2, -kFp8Max, kFp8Max);
+      c3 = __builtin_amdgcn_fmed3f(c3, -kFp8Max, kFp8Max);
+    }
     int word = __builtin_amdgcn_cvt_pk_fp8_f32(c0, c1, 0, false);
     word = __builtin_amdgcn_cvt_pk_fp8_f32(c2, c3, word, true);
     out[w] = (uint32_t)word;
@@ -205,17 +223,17 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
       vf[2 * e + 1] = bf16_to_f32(vr[e] >> 16);
     }
     float ks, vs;
-    if (a.kv_quant_mode == PA_QUANT_PER_TOKEN) {
-      float ka = 0.f, va = 0.f;
+    float ka = 0.f, va = 0.f;  // bounds of |x| in this thread's values (per-token scales: in the token's row)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        ka = fmaxf(ka, fabsf(kf[e]));
-        va = fmaxf(va, fabsf(vf[e]));
-      }
+    for (int e = 0; e < 8; ++e) {
+      ka = fmaxf(ka, fabsf(kf[e]));
+      va = fmaxf(va, fabsf(vf[e]));
+    }
+    if (a.kv_quant_mode == PA_QUANT_PER_TOKEN) {
       ka = row16_max(ka);  // the 16 lanes of a token
       va = row16_max(va);
-      ks = ka > 0.f ? __fdiv_rn(ka, kFp8Max) : 1.f;
-      vs = va > 0.f ? __fdiv_rn(va, kFp8Max) : 1.f;
+      ks = ka > 0.f ? bf16_amax_to_scale(ka) : 1.f;
+      vs = va > 0.f ? bf16_amax_to_scale(va) : 1.f;
       if (on && c == 0) {
         const int64_t so = block * a.stride_scale_b + h * a.stride_scale_h + off0 + tk;
         a.key_scale[so] = ks;
@@ -228,8 +246,13 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
       ks = vs = 1.f;
     }
     u32x2 kq, vq;
-    quantize8(kf, ks, kq);
-    quantize8(vf, vs, vq);
+    if (a.kv_quant_mode == PA_QUANT_PER_TOKEN && ka <= 0x1.fffffep127f && va <= 0x1.fffffep127f) {
+      quantize8<false>(kf, ks, ka, kq);
+      quantize8<false>(vf, vs, va, vq);
+    } else {
+      quantize8<true>(kf, ks, ka, kq);
+      quantize8<true>(vf, vs, va, vq);
+    }
     // K: lanes c, c+1 hold the two halves of one 16-byte (chunk, token) cell; the even one stores it
     const uint32_t p0 = dpp_u32<kDppSwap1>(kq[0]), p1 = dpp_u32<kDppSwap1>(kq[1]);
     if (on) {
@@ -259,9 +282,10 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
 
 // a group of n tokens from token t_first on, landing at slot0 .. slot0 + n - 1, for kv heads h0 .. h0 + nh - 1
 template <bool TO_FP8>
-__device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_first, int n, long long slot0, int h0, int nh,
-                                            int tid, uint8_t (*s_v)[256]) {
-  const long long block = slot0 / a.block_size;
+__device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_first, int n, long long slot0, int bs_shift,
+                                            int h0, int nh, int tid, uint8_t (*s_v)[256]) {
+  // bs_shift: log2 of the block size when that is a power of two (no 64-bit division then), else -1
+  const long long block = bs_shift >= 0 ? slot0 >> bs_shift : slot0 / a.block_size;
   const int off0 = (int)(slot0 - block * a.block_size);
   const int tk = tid >> 4, c = tid & 15;
   u32x4 kr[kHeadsPerWorkgroup], vr[kHeadsPerWorkgroup];
@@ -288,7 +312,7 @@ __device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_
 // in id order, so with `regroup` set the window a workgroup takes is chosen such that the eight windows of a
 // 128-token stretch are the next eight workgroups of ONE XCD.  The grid is then a multiple of 64 windows.
 template <bool TO_FP8>
-__global__ __launch_bounds__(256) void kv_cache_write_tile_kernel(const PaKvWriteArgs a, const int regroup) {
+__global__ __launch_bounds__(256) void kv_cache_write_tile_kernel(const PaKvWriteArgs a, const int regroup, const int bs_shift) {
   __shared__ long long s_slot[33];  // slots of tokens t0-1 .. t0+31
   __shared__ __attribute__((aligned(16))) uint8_t s_v[16][256];
   const int tid = threadIdx.x;
@@ -335,7 +359,7 @@ __global__ __launch_bounds__(256) void kv_cache_write_tile_kernel(const PaKvWrit
     const int j = __builtin_ctz(own);
     own &= own - 1;
     const int n = __builtin_ctzll(breaks >> (j + 1)) + 1;
-    write_group<TO_FP8>(a, t0 + j, n, s_slot[j + 1], h0, nh, tid, s_v);
+    write_group<TO_FP8>(a, t0 + j, n, s_slot[j + 1], bs_shift, h0, nh, tid, s_v);
   }
 }
 
@@ -472,13 +496,14 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
                         a->block_size % 16 == 0;
   if (rows_16b && a->num_tokens >= 2048 && a->num_kv_heads <= 65535) {
     const int regroup = a->block_size > 16;
+    const int bs_shift = (a->block_size & (a->block_size - 1)) == 0 ? __builtin_ctz((unsigned)a->block_size) : -1;
     long long windows = (a->num_tokens + 15) / 16;
     if (regroup) windows = (windows + 63) / 64 * 64;
     const dim3 grid((unsigned)windows, (unsigned)((a->num_kv_heads + kHeadsPerWorkgroup - 1) / kHeadsPerWorkgroup));
     if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
-      hipLaunchKernelGGL(kv_cache_write_tile_kernel<true>, grid, dim3(256), 0, stream, *a, regroup);
+      hipLaunchKernelGGL(kv_cache_write_tile_kernel<true>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
     else
-      hipLaunchKernelGGL(kv_cache_write_tile_kernel<false>, grid, dim3(256), 0, stream, *a, regroup);
+      hipLaunchKernelGGL(kv_cache_write_tile_kernel<false>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
   } else if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN) {
     hipLaunchKernelGGL(kv_cache_write_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
   } else {
