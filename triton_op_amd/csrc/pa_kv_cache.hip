@@ -178,7 +178,10 @@ __device__ __forceinline__ void quantize8(const float (&x)[8], float s, float xb
 // A workgroup owns the groups that START among its 16 tokens (a group may reach into the next workgroup's
 // tokens, which then skips them); with more than four groups among its tokens (scattered slots) it writes its
 // tokens one by one like the kernel above.
-constexpr int kHeadsPerWorkgroup = 4;  // kv heads one workgroup of the tile kernel walks, their rows all requested first
+// HPW: kv heads one workgroup of the tile kernel walks, their rows all requested first.  Measured on 262,144 tokens
+// x 8 heads: with per-token scales (more arithmetic per row between the loads and the stores) 2 heads per
+// workgroup beat 4 (block 16: 333 against 344 us, block 1024: 343 against 351 us); with per-tensor scales or a
+// 16-bit cache 4 are as good or better (block 16, per tensor: 327 against 350 us); 1 and 8 lose everywhere.
 
 // one kv head of a group: kr, vr are this thread's 16 bytes of the token's K and V row
 template <bool TO_FP8>
@@ -281,16 +284,16 @@ __device__ __forceinline__ void write_group_head(const PaKvWriteArgs& a, int n, 
 }
 
 // a group of n tokens from token t_first on, landing at slot0 .. slot0 + n - 1, for kv heads h0 .. h0 + nh - 1
-template <bool TO_FP8>
+template <bool TO_FP8, int HPW>
 __device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_first, int n, long long slot0, int bs_shift,
                                             int h0, int nh, int tid, uint8_t (*s_v)[256]) {
   // bs_shift: log2 of the block size when that is a power of two (no 64-bit division then), else -1
   const long long block = bs_shift >= 0 ? slot0 >> bs_shift : slot0 / a.block_size;
   const int off0 = (int)(slot0 - block * a.block_size);
   const int tk = tid >> 4, c = tid & 15;
-  u32x4 kr[kHeadsPerWorkgroup], vr[kHeadsPerWorkgroup];
+  u32x4 kr[HPW], vr[HPW];
 #pragma unroll
-  for (int i = 0; i < kHeadsPerWorkgroup; ++i) {
+  for (int i = 0; i < HPW; ++i) {
     kr[i] = vr[i] = u32x4{0, 0, 0, 0};
     if (tk < n && i < nh) {  // the rows are read once: non-temporal
       const long long t = t_first + tk;
@@ -301,7 +304,7 @@ __device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_
     }
   }
 #pragma unroll
-  for (int i = 0; i < kHeadsPerWorkgroup; ++i) {
+  for (int i = 0; i < HPW; ++i) {
     if (i < nh) write_group_head<TO_FP8>(a, n, block, off0, h0 + i, tid, kr[i], vr[i], s_v);
   }
 }
@@ -311,21 +314,30 @@ __device__ __forceinline__ void write_group(const PaKvWriteArgs& a, long long t_
 // through the same L2 close together.  Workgroups go to the eight XCDs (each with an L2 of its own) round robin
 // in id order, so with `regroup` set the window a workgroup takes is chosen such that the eight windows of a
 // 128-token stretch are the next eight workgroups of ONE XCD.  The grid is then a multiple of 64 windows.
-template <bool TO_FP8>
+template <bool TO_FP8, int HPW>
 __global__ __launch_bounds__(256) void kv_cache_write_tile_kernel(const PaKvWriteArgs a, const int regroup, const int bs_shift) {
   __shared__ long long s_slot[33];  // slots of tokens t0-1 .. t0+31
   __shared__ __attribute__((aligned(16))) uint8_t s_v[16][256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  long long window = blockIdx.x;
+  // workgroup id -> (16-token window, group of kv heads), the head groups of a window next to each other: they
+  // read the two halves of the same token rows and write neighbouring parts of the same pages
+  const int head_groups = (a.num_kv_heads + HPW - 1) / HPW;
+  long long window;
+  int hg;
   if (regroup) {
-    const long long q = window >> 3, xcd = window & 7;
-    window = (((q >> 3) << 3) + xcd) * 8 + (q & 7);
+    const long long q = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+    const long long unit = ((q >> 3) << 3) + xcd;  // (128-token stretch, head group): eight turns of one XCD
+    window = unit / head_groups * 8 + (q & 7);
+    hg = (int)(unit % head_groups);
+  } else {
+    window = blockIdx.x / head_groups;
+    hg = (int)(blockIdx.x % head_groups);
   }
   const long long t0 = window * 16;
   if (t0 >= a.num_tokens) return;
-  const int h0 = blockIdx.y * kHeadsPerWorkgroup;
-  const int nh = min(kHeadsPerWorkgroup, a.num_kv_heads - h0);
+  const int h0 = hg * HPW;
+  const int nh = min(HPW, a.num_kv_heads - h0);
   if (tid < 33) {
     const long long t = t0 - 1 + tid;
     s_slot[tid] = (t >= 0 && t < a.num_tokens) ? a.slot_mapping[t] : -1;
@@ -359,7 +371,7 @@ __global__ __launch_bounds__(256) void kv_cache_write_tile_kernel(const PaKvWrit
     const int j = __builtin_ctz(own);
     own &= own - 1;
     const int n = __builtin_ctzll(breaks >> (j + 1)) + 1;
-    write_group<TO_FP8>(a, t0 + j, n, s_slot[j + 1], bs_shift, h0, nh, tid, s_v);
+    write_group<TO_FP8, HPW>(a, t0 + j, n, s_slot[j + 1], bs_shift, h0, nh, tid, s_v);
   }
 }
 
@@ -494,16 +506,22 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
                         ((reinterpret_cast<uintptr_t>(a->key_cache) | reinterpret_cast<uintptr_t>(a->value_cache)) & 15) == 0 &&
                         a->stride_kc_b % 16 == 0 && a->stride_kc_h % 16 == 0 && a->stride_vc_b % 16 == 0 && a->stride_vc_h % 16 == 0 &&
                         a->block_size % 16 == 0;
-  if (rows_16b && a->num_tokens >= 2048 && a->num_kv_heads <= 65535) {
+  if (rows_16b && a->num_tokens >= 2048) {
     const int regroup = a->block_size > 16;
     const int bs_shift = (a->block_size & (a->block_size - 1)) == 0 ? __builtin_ctz((unsigned)a->block_size) : -1;
     long long windows = (a->num_tokens + 15) / 16;
     if (regroup) windows = (windows + 63) / 64 * 64;
-    const dim3 grid((unsigned)windows, (unsigned)((a->num_kv_heads + kHeadsPerWorkgroup - 1) / kHeadsPerWorkgroup));
-    if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
-      hipLaunchKernelGGL(kv_cache_write_tile_kernel<true>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
+    const bool per_token = a->cache_dtype == PA_DTYPE_FP8_E4M3FN && a->kv_quant_mode == PA_QUANT_PER_TOKEN;
+    const int hpw = per_token ? 2 : 4;
+    const long long head_groups = (a->num_kv_heads + hpw - 1) / hpw;
+    if (windows * head_groups > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+    const dim3 grid((unsigned)(windows * head_groups));
+    if (per_token)
+      hipLaunchKernelGGL((kv_cache_write_tile_kernel<true, 2>), grid, dim3(256), 0, stream, *a, regroup, bs_shift);
+    else if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
+      hipLaunchKernelGGL((kv_cache_write_tile_kernel<true, 4>), grid, dim3(256), 0, stream, *a, regroup, bs_shift);
     else
-      hipLaunchKernelGGL(kv_cache_write_tile_kernel<false>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
+      hipLaunchKernelGGL((kv_cache_write_tile_kernel<false, 4>), grid, dim3(256), 0, stream, *a, regroup, bs_shift);
   } else if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN) {
     hipLaunchKernelGGL(kv_cache_write_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
   } else {
