@@ -191,6 +191,8 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row_ok)
     rscale *= a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
   i32x8 qhi, qlo;
+  // an FP8 query times a power of two is its own FP8 head: the residual is zero and its MFMAs are skipped
+  const bool q_has_residual = a.query_dtype == PA_DTYPE_BF16;
   {
     const char* q_ptr = (const char*)a.query;
     const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (row_ok ? row : 0)) * a.stride_q_h;
@@ -255,7 +257,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
       const i32x8 ka = {(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
       s[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
       s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi, s[jj], 0, 0, 0, 0, 0, 0);
-      s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[jj], 0, 0, 0, 0, 0, 0);
+      if (q_has_residual) s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[jj], 0, 0, 0, 0, 0, 0);
     }
     // P is produced already multiplied by pmul = 256 / v_run (per-token V scales: v_run is the running
     // maximum of the scales, P then also carries v_scale / v_run <= 1 and the accumulator is kept in units
