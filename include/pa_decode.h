@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define PA_DECODE_ABI_VERSION 3
+#define PA_DECODE_ABI_VERSION 4
 /* Smallest useful size of the optional device workspace.  Its first 64 bytes hold a work-item counter: with
  * it, batches with per-sequence query lengths are launched as a resident grid that pulls live (sequence,
  * partition, row tile, head) items from the counter instead of one workgroup per possible item.  These 64
@@ -56,7 +56,8 @@ enum {
   PA_ERR_UNSUPPORTED = -3,    /* dtype / head size / block size / group size not supported */
   PA_ERR_BAD_SHAPE = -4,      /* non-positive size, bad partition size, stride the kernels cannot take */
   PA_ERR_LAUNCH = -5,         /* the HIP runtime refused the launch (see pa_decode_last_hip_error) */
-  PA_ERR_NO_DEVICE = -6
+  PA_ERR_NO_DEVICE = -6,
+  PA_ERR_SCRATCH_TOO_SMALL = -7 /* pa_decode_noalloc: the call's buffers exceed PA_DECODE_NOALLOC_SCRATCH_BYTES */
 };
 
 /*
@@ -172,6 +173,27 @@ int pa_decode_reduce(const PaDecodeArgs* args, void* hip_stream);
 /* Both stages back to back on one stream: the body of the reference's paged_attention_decode.  Stage 2
  * skips the sequences stage 1 has finished, and is not launched when max_num_partitions == 1 (no sinks). */
 int pa_decode(const PaDecodeArgs* args, void* hip_stream);
+
+/*
+ * pa_decode for callers that cannot allocate device memory and have no partition buffers to pass: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose entry point allocates its three buffers with torch.zeros on every call,
+ * pa_decode_triton_gluon_fp8.py:1726-1733).  args is filled as for pa_decode, except that exp_sums, max_logits,
+ * tmp_output and workspace must be NULL and workspace_bytes 0 (the strides of the partition buffers are
+ * ignored): the library places all four in a device array of PA_DECODE_NOALLOC_SCRATCH_BYTES that it holds on
+ * every GPU it runs on until the process ends, and calls no hipMalloc, hipFree or other allocating routine.
+ * Bytes needed, each term rounded up to a multiple of 256, with n = num_seqs * num_kv_heads *
+ * max_num_partitions * q_len * group_size:
+ *     pa_decode_workspace_bytes(num_seqs, max_num_partitions) + 4 n + 4 n + 2 n * head_size;
+ * a call that needs more returns PA_ERR_SCRATCH_TOO_SMALL and launches nothing (choose a larger partition_size,
+ * as pa_decode_select_partition_size does, or use pa_decode with buffers of your own).  The partition buffers
+ * are not handed back.  All calls on one GPU share that GPU's array: calls that may overlap on the GPU (two
+ * streams, two threads) race; calls on one stream, or ordered by events, do not.  The array keeps the last
+ * call's contents; the call clears the counters it needs zero with a small kernel (no memset node, so it can be
+ * captured into a graph) and ignores PA_DECODE_FLAG_REUSE_ITEM_LIST.
+ */
+#define PA_DECODE_NOALLOC_SCRATCH_BYTES (64u << 20)
+int pa_decode_noalloc(const PaDecodeArgs* args, void* hip_stream);
 
 /*
  * KV-cache write: the step before the decode path.  Writes num_tokens new (key, value) rows

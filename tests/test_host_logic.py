@@ -60,7 +60,7 @@ def test_workspace_size_rule(pa_lib):
 
 def test_error_strings_and_null_arguments(pa_lib):
     assert pa_lib.pa_decode_error_string(0) == b"ok"
-    for code in range(-6, 0):
+    for code in range(-7, 0):
         assert pa_lib.pa_decode_error_string(code) not in (b"ok", b"unknown error code")
     assert pa_lib.pa_decode(None, None) == -1
     a = _cabi.PaDecodeArgs()
@@ -68,6 +68,12 @@ def test_error_strings_and_null_arguments(pa_lib):
     a.struct_size = C.sizeof(_cabi.PaDecodeArgs)
     assert pa_lib.pa_decode_partition(C.byref(a), None) == -1  # buffers are NULL
     assert pa_lib.pa_debug_fp8_decode(None, None, 4, None) == -1
+    assert pa_lib.pa_decode_noalloc(None, None) == -1
+    b = _cabi.PaDecodeArgs()
+    assert pa_lib.pa_decode_noalloc(C.byref(b), None) == -2
+    b.struct_size = C.sizeof(_cabi.PaDecodeArgs)
+    b.workspace_bytes = 64  # this entry point owns the workspace and the partition buffers: passing one is an error
+    assert pa_lib.pa_decode_noalloc(C.byref(b), None) == -4
 
 
 def test_partition_size_choices():

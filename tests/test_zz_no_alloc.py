@@ -1,0 +1,74 @@
+"""pa_decode_noalloc, the entry point that allocates nothing: its output must equal pa_decode's bit for bit (the
+same kernels run on the same inputs; only where the partition buffers live differs), on two calls in a row that
+share the library's scratch array, the second with a smaller input, and a call too large for the array must be
+refused before anything is launched."""
+import ctypes as C
+
+import pytest
+import torch
+
+import triton_op_amd as T
+from triton_op_amd import _cabi
+from triton_op_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _plan(wl, out, partition_size):
+    return T.plan_decode(out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                         wl.softmax_scale, wl.q_len, wl.max_context_len, torch.bfloat16, None, wl.key_scale,
+                         wl.value_scale, partition_size=partition_size, query_lens=wl.q_lens)
+
+
+def _workloads(dev):
+    # first a ragged MTP batch over per-token scales (shared-stream kernel, sorted dispatch, listed reduce, the
+    # queue counters), then a smaller one on the other partition kernel with several partitions per sequence
+    g = torch.Generator().manual_seed(11)
+    ctx_a = torch.randint(16, 2560, (200,), generator=g, dtype=torch.int32)
+    ql_a = torch.randint(1, 4, (200,), generator=g, dtype=torch.int32)
+    a = W.make_decode_workload(name="noalloc_a", seed=21, batch=200, num_q_heads=32, num_kv_heads=2, block_size=16,
+                               context_lens=ctx_a, q_len=3, q_lens=ql_a, scale_mode="token").to(dev)
+    ctx_b = torch.tensor([1500, 17, 700], dtype=torch.int32)
+    b = W.make_decode_workload(name="noalloc_b", seed=22, batch=3, num_q_heads=16, num_kv_heads=2, block_size=16,
+                               context_lens=ctx_b, q_len=1).to(dev)
+    return [(a, 256), (b, 256)]
+
+
+def test_noalloc_matches_pa_decode_on_two_calls_in_a_row():
+    dev = torch.device("cuda:0")
+    lib = _cabi.load_library()
+    stream = torch.cuda.current_stream(dev)
+    for wl, ps in _workloads(dev):
+        print(f"[noalloc] {wl.name} batch={wl.batch} partition_size={ps}", flush=True)
+        ref = torch.full_like(wl.query, float("nan"))
+        _plan(wl, ref, ps).run()
+        out = torch.full_like(wl.query, float("nan"))
+        plan = _plan(wl, out, ps)
+        # poison this plan's own buffers: the entry point must not touch them
+        plan.tmp_output.fill_(float("nan"))
+        plan.exp_sums.fill_(float("nan"))
+        before = torch.cuda.memory_allocated(dev)
+        plan.run_noalloc(stream.cuda_stream)
+        assert torch.cuda.memory_allocated(dev) == before
+        torch.cuda.synchronize()
+        assert not torch.isnan(out.float()).any()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), wl.name
+        assert torch.isnan(plan.tmp_output.float()).all() and torch.isnan(plan.exp_sums).all()
+
+
+def test_noalloc_refuses_what_does_not_fit():
+    dev = torch.device("cuda:0")
+    lib = _cabi.load_library()
+    wl = W.make_decode_workload(name="noalloc_big", seed=23, batch=2, num_q_heads=8, num_kv_heads=1, block_size=16,
+                                context_lens=torch.tensor([64, 33], dtype=torch.int32), q_len=1).to(dev)
+    out = torch.full_like(wl.query, 7.0)
+    plan = _plan(wl, out, 256)
+    a = _cabi.PaDecodeArgs.from_buffer_copy(plan.args)
+    a.exp_sums = a.max_logits = a.tmp_output = a.workspace = None
+    a.workspace_bytes = 0
+    # claim a partition axis whose buffers would take more than the scratch array: 2 * 1 * P * 8 rows * 264 B
+    a.max_num_partitions = _cabi.PA_DECODE_NOALLOC_SCRATCH_BYTES // (2 * 8 * 264) + 1
+    rc = lib.pa_decode_noalloc(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == _cabi.PA_ERR_SCRATCH_TOO_SMALL
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.full_like(out, 7.0))  # nothing ran

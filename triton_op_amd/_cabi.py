@@ -12,8 +12,10 @@ import threading
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
-PA_DECODE_ABI_VERSION = 3
+PA_DECODE_ABI_VERSION = 4
 PA_DECODE_WORKSPACE_BYTES = 64
+PA_DECODE_NOALLOC_SCRATCH_BYTES = 64 << 20
+PA_ERR_SCRATCH_TOO_SMALL = -7
 PA_DECODE_FLAG_REUSE_ITEM_LIST = 1
 PA_DTYPE_BF16, PA_DTYPE_FP8_E4M3FN = 0, 1
 PA_QUANT_NONE, PA_QUANT_PER_TENSOR, PA_QUANT_PER_TOKEN = -1, 0, 1
@@ -28,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "pa_decode_partition",
     "pa_decode_reduce",
     "pa_decode",
+    "pa_decode_noalloc",
     "pa_debug_fp8_decode",
     "pa_kv_cache_write",
     "pa_quantize_kv_cache",
@@ -97,7 +100,7 @@ def load_library(path: str = None) -> C.CDLL:
         lib.pa_decode_workspace_bytes.argtypes = [C.c_int32, C.c_int32]
         lib.pa_decode_select_partition_size.restype = C.c_int
         lib.pa_decode_select_partition_size.argtypes = [C.c_int32] * 6
-        for name in ("pa_decode_partition", "pa_decode_reduce", "pa_decode"):
+        for name in ("pa_decode_partition", "pa_decode_reduce", "pa_decode", "pa_decode_noalloc"):
             fn = getattr(lib, name)
             fn.restype = C.c_int
             fn.argtypes = [C.POINTER(PaDecodeArgs), C.c_void_p]

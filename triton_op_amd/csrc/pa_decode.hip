@@ -12,6 +12,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "../../include/pa_decode.h"
 #include "pa_common.h"
 #include "pa_partition_kernel.h"
@@ -19,7 +21,18 @@
 #include "pa_plan_kernel.h"
 #include "pa_reduce_kernel.h"
 
+// Scratch of pa_decode_noalloc, the entry point for callers that can neither allocate nor pass partition buffers:
+// the item-list workspace and the three partition buffers of one call.  Every GPU the library runs on holds its
+// own copy at its own address; host code reaches it only through the address hipGetSymbolAddress returns there.
+static __device__ __align__(256) unsigned char scratch[PA_DECODE_NOALLOC_SCRATCH_BYTES];
+
 namespace {
+
+// the first `n` int32 words at p become zero (a launch, not a memset node: callers may be capturing a graph)
+__global__ void pa_clear_words_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
 
 __global__ void pa_fp8_decode_kernel(const uint8_t* codes, float* out, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -297,6 +310,7 @@ const char* pa_decode_error_string(int code) {
     case PA_ERR_BAD_SHAPE: return "bad size, partition size or stride";
     case PA_ERR_LAUNCH: return "HIP launch failed";
     case PA_ERR_NO_DEVICE: return "no HIP device";
+    case PA_ERR_SCRATCH_TOO_SMALL: return "the call's partition buffers do not fit the library's scratch array";
   }
   return "unknown error code";
 }
@@ -437,6 +451,73 @@ int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
     return launch_reduce_listed(a, hip_stream);
   }
   return launch_reduce(a, hip_stream, true);
+}
+
+int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
+  if (!a) return PA_ERR_NULL_POINTER;
+  if (a->struct_size != sizeof(PaDecodeArgs)) return PA_ERR_BAD_STRUCT;
+  // the library owns these four in this entry point: a caller that passes its own wants pa_decode
+  if (a->exp_sums || a->max_logits || a->tmp_output || a->workspace || a->workspace_bytes) return PA_ERR_BAD_SHAPE;
+  if (a->num_seqs <= 0 || a->num_kv_heads <= 0 || a->group_size <= 0 || a->q_len <= 0 || a->max_num_partitions <= 0 ||
+      a->head_size != kHeadSize)
+    return PA_ERR_BAD_SHAPE;
+
+  // ---- this device's copy of the scratch array: its address is asked for once per device, with that device current
+  constexpr int kMaxDevices = 64;
+  static unsigned char* scratch_of_device[kMaxDevices] = {};
+  static std::mutex scratch_lock;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return PA_ERR_NO_DEVICE;
+  unsigned char* base;
+  {
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_of_device[dev]) {
+      void* p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !p) {
+        g_last_hip_error = (int)e;
+        return PA_ERR_LAUNCH;
+      }
+      scratch_of_device[dev] = static_cast<unsigned char*>(p);
+    }
+    base = scratch_of_device[dev];
+  }
+
+  // ---- layout: workspace, max_logits, exp_sums, tmp_output, each at a multiple of 256 bytes ------------------
+  const auto round256 = [](long long n) { return (n + 255) / 256 * 256; };
+  const long long ge = (long long)a->q_len * a->group_size;
+  const long long rows = (long long)a->num_seqs * a->num_kv_heads * a->max_num_partitions * ge;
+  const long long ws_bytes = full_workspace_bytes(a->num_seqs, a->max_num_partitions);
+  const long long off_ml = round256(ws_bytes);
+  const long long off_es = off_ml + round256(4 * rows);
+  const long long off_tmp = off_es + round256(4 * rows);
+  const long long total = off_tmp + round256(2 * rows * kHeadSize);
+  if (total > (long long)PA_DECODE_NOALLOC_SCRATCH_BYTES) return PA_ERR_SCRATCH_TOO_SMALL;
+
+  PaDecodeArgs k = *a;
+  k.workspace = reinterpret_cast<int32_t*>(base);
+  k.workspace_bytes = ws_bytes;
+  k.max_logits = reinterpret_cast<float*>(base + off_ml);
+  k.exp_sums = reinterpret_cast<float*>(base + off_es);
+  k.tmp_output = base + off_tmp;
+  k.stride_es_p = ge;
+  k.stride_es_h = ge * a->max_num_partitions;
+  k.stride_es_s = k.stride_es_h * a->num_kv_heads;
+  k.stride_tmp_g = kHeadSize;
+  k.stride_tmp_p = ge * kHeadSize;
+  k.stride_tmp_h = k.stride_tmp_p * a->max_num_partitions;
+  k.stride_tmp_s = k.stride_tmp_h * a->num_kv_heads;
+  // the array keeps the last call's contents (a call that was cut short may have left its counters non-zero, and
+  // an item list of another batch): the counters are cleared, the lists are rebuilt
+  k.flags &= ~PA_DECODE_FLAG_REUSE_ITEM_LIST;
+  hipLaunchKernelGGL(pa_clear_words_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(hip_stream),
+                     k.workspace, kPlanHeaderWords);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return PA_ERR_LAUNCH;
+  }
+  return pa_decode(&k, hip_stream);
 }
 
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream) {

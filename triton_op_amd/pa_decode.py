@@ -80,6 +80,18 @@ class DecodePlan:
             stream = torch.cuda.current_stream(self.output.device).cuda_stream
         _cabi.check(self._lib.pa_decode(C.byref(self.args), C.c_void_p(stream)), "pa_decode")
 
+    def run_noalloc(self, stream: Optional[int] = None) -> None:
+        """The same call through `pa_decode_noalloc`: the partition buffers and the workspace of this plan are
+        left alone, the library uses its own per-GPU scratch array instead (64 MiB; larger calls raise).  Calls
+        that may overlap on one GPU share that array and race."""
+        if stream is None:
+            stream = torch.cuda.current_stream(self.output.device).cuda_stream
+        a = PaDecodeArgs.from_buffer_copy(self.args)
+        a.exp_sums = a.max_logits = a.tmp_output = a.workspace = None
+        a.workspace_bytes = 0
+        a.flags = 0
+        _cabi.check(self._lib.pa_decode_noalloc(C.byref(a), C.c_void_p(stream)), "pa_decode_noalloc")
+
     def run_partition(self, stream: Optional[int] = None) -> None:
         if stream is None:
             stream = torch.cuda.current_stream(self.output.device).cuda_stream
