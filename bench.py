@@ -1,18 +1,29 @@
 #!/usr/bin/env python3
 """Benchmark of the paged-attention decode hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--partition-size N]
-    python bench.py --workload kv_write | kv_quantize      (the KV-cache write kernels, the step before the path)
+    python bench.py [--gpus 1] [--steps K] [--warmup W]            the headline (c2) plus the other configurations
+    python bench.py --workload c1|c2|c3|c4|c5 [--partition-size N]   one configuration
+    python bench.py --workload ref:B,Hq,Hkv,bs,qlen[,transv][,ctx=N]  one row of the reference harness's sweep
+    python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1]
+    python bench.py --workload probe_gather                          read-only probe of c2's page-gather pattern
+    python bench.py --workload kv_write | kv_quantize                the KV-cache write kernels, the step before the path
 
-A step is one call of the op (partition kernel + reduce kernel on one stream) on one batch of
-synthetic input that is already resident in HBM.  Consecutive steps use different KV pools so the
-256 MB Infinity Cache cannot serve the KV stream.  Prints ONE JSON line.
+A step is one call of the op (partition kernel + reduce kernel on one stream) on one batch of synthetic input
+that is already resident in HBM.  Consecutive steps use different KV pools so the 256 MB last-level cache
+cannot serve the KV stream.  Prints ONE JSON line.
+
+`ref:` builds the inputs the reference harness builds (test_pa_mtp.py:660-722,763-783): uniform(-1,1) bf16 query
+and cache, a pool of 16384 tokens' worth of pages per sequence, block tables drawn with replacement, the cache
+quantised per (block, head, token), the query per row (FP8 query with per-row scales: the Gluon entry point's
+contract), context length 4096 unless given.  Every decode line also carries the reference's own bandwidth figure
+(test_pa_mtp.py:937-945: K, V, query and output bytes over the time, in units of 1.024^4 * 1e12 B/s).
 """
 from __future__ import annotations
 
 import argparse
 import ctypes as C
 import json
+import math
 import os
 import sys
 import time
@@ -23,35 +34,273 @@ if HERE not in sys.path:
 
 METRIC = "µs/call + achieved KV HBM GB/s (% peak), FP8 KV, B=64 GQA8 ctx=4k"
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the partition kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
-# the counter reads for a plain copy of known size (profiles/pa_partition_kernel_c2_hbm_traffic.md,
-# profiles/pa_partition_shared_kernel_c5_hbm_traffic.md); keyed by (workload, partition size) because the
-# partial-output traffic depends on the partitioning
-HBM_TRAFFIC_BYTES = {("c2_fp8_b64_ctx4k", 4096): 541_400_000, ("c5_ragged_mix", 7424): 2_050_400_000}
+SETTLE_CALLS = 100  # untimed calls before anything is measured (clocks and power state settle), not part of --warmup
+
+# HBM bytes per launch of the partition kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# counter reads for a plain copy of known size.  An entry holds for ONE (workload, partition size, launch) as
+# pa_decode_launch_info names it: when the launch layer or a kernel's instantiation changes, the figure is stale and
+# the line carries null and a note instead.
+HBM_TRAFFIC = {
+    ("c2_fp8_b64_ctx4k", 4096): {
+        "bytes": 541_400_000, "launch": "pa_partition_kernel<fp8, bs16, 4 waves> x 512",
+        "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
+    ("c5_ragged_mix", 7424): {
+        "bytes": 2_050_400_000,
+        "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 6512, sorted items",
+        "profile": "profiles/pa_partition_shared_kernel_c5_hbm_traffic.md"},
+}
 
 
-def _partition_kernel_name(wl):
-    """The kernel the library launches for this workload: more than 16 query rows per kv head over an FP8
-    cache go to the kernel whose row tiles share one pass over the pages."""
-    ge = wl.q_len * (wl.num_q_heads // wl.num_kv_heads)
-    fp8 = wl.key_cache.element_size() == 1
-    return "pa_partition_shared_kernel" if (fp8 and ge > 16) else "pa_partition_kernel"
+# ---------------------------------------------------------------------------------------------------------------
+# workloads
+# ---------------------------------------------------------------------------------------------------------------
+def _parse_kv(text):
+    out = {}
+    for item in text.split(","):
+        if not item:
+            continue
+        k, _, v = item.partition("=")
+        out[k.strip()] = v.strip()
+    return out
 
 
-def _cpu_baseline(wl_cpu_sample, n_seq_sample, target_seconds=20.0):
+def _make_ref_workload(spec, device, seed):
+    """One row of the reference harness's sweep, inputs made as the harness makes them."""
+    import torch
+
+    import triton_op_amd as T
+    from triton_op_amd import kv_layout as L
+    from triton_op_amd.workloads import Workload
+
+    parts = spec.split(",")
+    b, hq, hkv, bs, qlen = (int(x) for x in parts[:5])
+    transv, ctx = False, 4096
+    for x in parts[5:]:
+        if x == "transv":
+            transv = True
+        elif x.startswith("ctx="):
+            ctx = int(x[4:])
+        else:
+            raise ValueError(f"ref: unknown field {x!r}")
+    d = 128
+    blocks_per_seq = (ctx + bs - 1) // bs
+    total_blocks = ((16384 + bs - 1) // bs) * b
+    gen = torch.Generator(device=device).manual_seed(seed)
+    kc16, vc16 = L.create_kv_cache(total_blocks, bs, hkv, d, torch.bfloat16, generator=gen, device=device)
+    kq, _, vq, _, ks, vs = T.quantize_kv_cache_symmetric(kc16, vc16, torch.float8_e4m3fn)
+    del kc16, vc16
+    if transv:
+        vq = L.shuffle_value_cache_layout(vq)
+    q_tok = torch.empty(b * qlen, hq, d, device=device).uniform_(-1.0, 1.0, generator=gen).to(torch.bfloat16)
+    q8, q8s = L.pertoken_quant(L.mtp_pack(q_tok, b, qlen, hkv).contiguous().float())
+    bt = torch.randint(0, total_blocks, (b, blocks_per_seq), generator=gen, device=device, dtype=torch.int32)
+    return Workload(
+        name=f"ref_b{b}_h{hq}x{hkv}_bs{bs}_q{qlen}{'_transv' if transv else ''}_ctx{ctx}", query=q8, key_cache=kq,
+        value_cache=vq, context_lens=torch.full((b,), ctx, dtype=torch.int32, device=device), block_tables=bt,
+        softmax_scale=1.0 / math.sqrt(d), q_len=qlen, q_lens=None, key_scale=ks, value_scale=vs, partition_size=256,
+        num_kv_heads=hkv, num_q_heads=hq, head_size=d, block_size=bs, max_context_len=ctx,
+        meta={"seed": seed, "pool_blocks": total_blocks, "kv_dtype": "fp8", "scale_mode": "token",
+              "query_scale": q8s.contiguous(), "distribution": "uniform(-1,1), block tables with replacement"})
+
+
+def _make_custom_workload(spec, device, seed):
+    import torch
+
+    from triton_op_amd import kv_layout as L
+    from triton_op_amd import workloads as W
+
+    kv = _parse_kv(spec)
+    b, hq, hkv = int(kv.get("b", 64)), int(kv.get("hq", 64)), int(kv.get("hkv", 8))
+    q, ctx, bs = int(kv.get("q", 1)), int(kv.get("ctx", 4096)), int(kv.get("bs", 16))
+    scale, kvd, qd = kv.get("scale", "tensor"), kv.get("kv", "fp8"), kv.get("qdtype", "bf16")
+    transv = kv.get("transv", "0") == "1"
+    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv"}
+    if unknown:
+        raise ValueError(f"custom: unknown keys {sorted(unknown)}")
+    wl = W.make_decode_workload(
+        name=f"custom_b{b}_h{hq}x{hkv}_bs{bs}_q{q}_ctx{ctx}_{kvd}_{scale}_{qd}q{'_transv' if transv else ''}", seed=seed,
+        batch=b, num_q_heads=hq, num_kv_heads=hkv, block_size=bs,
+        context_lens=torch.full((b,), ctx, dtype=torch.int32), q_len=q, kv_dtype=kvd,
+        scale_mode="none" if kvd == "bf16" else scale, device=device, transposed_v=transv)
+    if qd == "fp8":
+        q8, q8s = L.pertoken_quant(wl.query.float())
+        wl.query = q8
+        wl.meta["query_scale"] = q8s.contiguous()
+    return wl
+
+
+def _make_workload(name, device, pool_index, batch=None):
+    from triton_op_amd import workloads as W
+
+    if name.startswith("ref:"):
+        return _make_ref_workload(name[4:], device, 1234 + 100 * pool_index)
+    if name.startswith("custom:"):
+        return _make_custom_workload(name[7:], device, 77 + 100 * pool_index)
+    wl = W.make_config(name, device=device, batch=batch)
+    if pool_index:
+        # same shapes, different page contents and block tables
+        wl = W.make_decode_workload(
+            name=wl.name, seed=wl.meta["seed"] + 100 * pool_index, batch=wl.batch, num_q_heads=wl.num_q_heads,
+            num_kv_heads=wl.num_kv_heads, block_size=wl.block_size, context_lens=wl.context_lens.cpu(), q_len=wl.q_len,
+            q_lens=None if wl.q_lens is None else wl.q_lens.cpu(), kv_dtype=wl.meta["kv_dtype"],
+            scale_mode=wl.meta["scale_mode"], device=device)
+    return wl
+
+
+def _reference_bandwidth_tbps(wl, us):
+    """The reference harness's bandwidth figure (test_pa_mtp.py:937-945):
+    B*D*(2*ctx*Hkv*sizeof(kv) + 2*qlen*Hq*sizeof(q)) / (us * 1e6 * 1.024**4); sums over the batch when ragged."""
+    import torch
+
+    tokens = int(wl.context_lens.to(torch.int64).sum())
+    q_rows = int(wl.q_lens.to(torch.int64).sum()) if wl.q_lens is not None else wl.batch * wl.q_len
+    nbytes = wl.head_size * (2 * tokens * wl.num_kv_heads * wl.key_cache.element_size() +
+                             2 * q_rows * wl.num_q_heads * wl.query.element_size())
+    return nbytes / (us * 1e6 * 1.024 ** 4)
+
+
+def _dtype_text(wl):
+    kv = "fp8_e4m3fn" if wl.key_cache.element_size() == 1 else "bf16"
+    q = "fp8_e4m3fn" if wl.query.element_size() == 1 else "bf16"
+    if kv == "bf16":
+        return "bf16 KV and Q on bf16 MFMA, f32 accumulate and softmax, bf16 out"
+    return (f"{kv} KV on FP8 MFMA ({q} Q" + (" and P" if q != "bf16" else " and P, each") +
+            " carried as FP8 head + residual), f32 accumulate and softmax, bf16 out")
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# timing of one decode configuration
+# ---------------------------------------------------------------------------------------------------------------
+class _Config:
+    """`pools` independent copies of one workload with their validated plans."""
+
+    def __init__(self, name, dev, pools, partition_size=None, batch=None, shared_from=None):
+        import torch
+
+        import triton_op_amd as T
+
+        self.wls = shared_from.wls if shared_from is not None else [
+            _make_workload(name, dev, i, batch) for i in range(pools)]
+        self.plans = []
+        for wl in self.wls:
+            out = torch.empty(wl.query.shape, dtype=torch.bfloat16, device=dev)
+            self.plans.append(T.plan_decode(
+                out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
+                wl.q_len, wl.max_context_len, torch.bfloat16, wl.meta.get("query_scale"), wl.key_scale, wl.value_scale,
+                partition_size=partition_size or None, query_lens=wl.q_lens))
+        self.wl0 = self.wls[0]
+        self.kv_bytes = self.wl0.kv_bytes()
+        self.partition_size = int(self.plans[0].args.partition_size)
+        self.launch = self.plans[0].launch_info()
+        self.kernel = self.launch.split("<")[0]
+
+
+def _time_config(lib, cfg, stream, steps, warmup, settle):
+    """Returns the timings of one configuration.  Order: `settle` untimed calls; the partition kernel alone
+    (roofline); `warmup` untimed calls and exactly `steps` calls between two synchronisations (ms_per_step); the same
+    `steps` calls again with an event pair around each (median µs per call)."""
+    import torch
+
+    from triton_op_amd import _cabi
+
+    sh = C.c_void_p(stream.cuda_stream)
+    plans, n = cfg.plans, len(cfg.plans)
+
+    def call(i):
+        rc = lib.pa_decode(C.byref(plans[i % n].args), sh)
+        if rc:
+            _cabi.check(rc, "pa_decode")
+
+    for i in range(settle):
+        call(i)
+    torch.cuda.synchronize()
+
+    # ---- the dominant kernel alone.  When the partition kernel is the whole call (one partition per sequence), one
+    # event pair brackets `steps` back-to-back launches, which is what a kernel trace's average sees; otherwise other
+    # kernels run in between and every launch gets an event pair of its own (which also brackets its dispatch).
+    solo = plans[0].args.max_num_partitions == 1
+    if solo:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(steps):
+            rc = lib.pa_decode_partition(C.byref(plans[i % n].args), sh)
+            if rc:
+                _cabi.check(rc, "pa_decode_partition")
+        e1.record(stream)
+        torch.cuda.synchronize()
+        k_us_avg = e0.elapsed_time(e1) * 1e3 / steps
+        k_timing = f"one event pair around {steps} back-to-back launches"
+    else:
+        kevs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i in range(steps):
+            p = plans[i % n]
+            kevs[i][0].record(stream)
+            rc = lib.pa_decode_partition(C.byref(p.args), sh)
+            kevs[i][1].record(stream)
+            if rc:
+                _cabi.check(rc, "pa_decode_partition")
+            lib.pa_decode_reduce(C.byref(p.args), sh)
+        torch.cuda.synchronize()
+        k_us = [e0.elapsed_time(e1) * 1e3 for e0, e1 in kevs]
+        k_us_avg = sum(k_us) / len(k_us)
+        k_timing = "an event pair around every launch (planning kernel included when the launch uses one)"
+
+    # ---- the whole op
+    for i in range(warmup):
+        call(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        call(i)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for i in range(steps):
+        evs[i][0].record(stream)
+        call(i)
+        evs[i][1].record(stream)
+    torch.cuda.synchronize()
+    call_us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
+    return {"us_median": call_us[len(call_us) // 2], "us_mean": sum(call_us) / len(call_us), "wall_ms": wall_ms,
+            "kernel_us_avg": k_us_avg, "kernel_timing": k_timing}
+
+
+def _traffic(cfg):
+    entry = HBM_TRAFFIC.get((cfg.wl0.name, cfg.partition_size))
+    if entry is None:
+        return None, "no rocprofv3 FETCH_SIZE/WRITE_SIZE measurement on record for this workload and partition size"
+    if entry["launch"] != cfg.launch:
+        return None, (f"the figure on record ({entry['profile']}) was measured on '{entry['launch']}', "
+                      f"this run launches '{cfg.launch}'")
+    return entry["bytes"], entry["profile"]
+
+
+def _config_line(cfg, t):
+    """The short record of a configuration for the `configs` array of the headline line."""
+    achieved = cfg.kv_bytes / (t["kernel_us_avg"] * 1e-6) / 1e9
+    return {
+        "workload": cfg.wl0.name, "partition_size": cfg.partition_size, "us_per_call": round(t["us_median"], 2),
+        "kv_GBps": round(cfg.kv_bytes / (t["us_median"] * 1e-6) / 1e9, 1), "kernel": cfg.kernel, "launch": cfg.launch,
+        "kernel_us_avg": round(t["kernel_us_avg"], 2), "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_launch": cfg.kv_bytes,
+        "reference_formula_TBps": round(_reference_bandwidth_tbps(cfg.wl0, t["us_median"]), 3),
+    }
+
+
+def _cpu_baseline(wl, n_seq_sample, full_batch, target_seconds=20.0):
     """The torch restatement of the reference's own oracle (oracle/pa_oracle.py, following
     test_pa_mtp.py:223-291) timed on the host cores over a few sequences of the same workload."""
     import torch
 
     from oracle import pa_oracle as O
 
-    wl = wl_cpu_sample
     threads = torch.get_num_threads()
 
     def run(ids):
         return O.paged_attention_decode_oracle(
             wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
-            wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, seq_ids=ids)
+            wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, seq_ids=ids,
+            query_scale=wl.meta.get("query_scale"))
 
     run([0])  # warm-up
     t0, done = time.perf_counter(), 0
@@ -66,20 +315,174 @@ def _cpu_baseline(wl_cpu_sample, n_seq_sample, target_seconds=20.0):
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "us_per_call_extrapolated": round(dt / done * 1e6 * _FULL_BATCH[0], 1),
-        "sample": f"{done} single-sequence calls over the first {n_seq_sample} of {_FULL_BATCH[0]} sequences of "
+        "us_per_call_extrapolated": round(dt / done * 1e6 * full_batch, 1),
+        "sample": f"{done} single-sequence calls over the first {n_seq_sample} of {full_batch} sequences of "
                   f"the same workload, f32 torch ops, {dt:.1f} s wall on {threads} threads",
     }
 
 
-_FULL_BATCH = [0]
+def _device_copy_gbps(dev, stream):
+    import torch
+
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return 10 * 2 * (1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
+def _bench_decode(a) -> int:
+    import torch
+
+    from triton_op_amd import _cabi
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    lib = _cabi.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(dev)
+    stream = torch.cuda.current_stream(dev)
+
+    headline = a.workload or "c2"
+    cfg = _Config(headline, dev, a.pools, a.partition_size, a.batch or None)
+    t = _time_config(lib, cfg, stream, a.steps, a.warmup, SETTLE_CALLS)
+    wl0 = cfg.wl0
+    achieved = cfg.kv_bytes / (t["kernel_us_avg"] * 1e-6) / 1e9
+    traffic, traffic_note = _traffic(cfg)
+    value = cfg.kv_bytes / (t["us_median"] * 1e-6) / 1e9
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s (KV bytes / median µs per call)",
+        "us_per_call": round(t["us_median"], 2),
+        "us_per_call_mean": round(t["us_mean"], 2),
+        "pct_of_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 2),
+        "reference_formula_TBps": round(_reference_bandwidth_tbps(wl0, t["us_median"]), 3),
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "settle_calls": SETTLE_CALLS,
+        "ms_per_step": round(t["wall_ms"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": _dtype_text(wl0),
+        "data": "synthetic",
+        "config": {
+            "workload": wl0.name,
+            "batch": wl0.batch, "q_heads": wl0.num_q_heads, "kv_heads": wl0.num_kv_heads,
+            "head_size": wl0.head_size, "q_len": wl0.q_len, "block_size": wl0.block_size,
+            "context_len_max": wl0.max_context_len, "partition_size": cfg.partition_size,
+            "kv_bytes_per_call": cfg.kv_bytes, "kv_pools_rotated": len(cfg.plans), "device": props.name,
+            "compute_units": props.multi_processor_count,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": cfg.kernel,
+            "launch": cfg.launch,
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "traffic_note": traffic_note,
+            "kernel_us_avg": round(t["kernel_us_avg"], 2),
+            "kernel_timing": t["kernel_timing"],
+            "algorithmic_bytes_per_launch": cfg.kv_bytes,
+        },
+    }
+
+    # ---- the other configurations, driver-visible in the same line (the default run only) ----------------------
+    if not a.workload and not a.no_configs:
+        lines = []
+        # c2 at the configuration's literal partition size 256 (the reference's constant): same pools
+        c2_256 = _Config("c2", dev, a.pools, 256, shared_from=cfg)
+        lines.append(_config_line(c2_256, _time_config(lib, c2_256, stream, min(a.steps, 30), 5, 30)))
+        del c2_256
+        for name in ("c3", "c4", "c5"):
+            other = _Config(name, dev, 1)  # each of them streams far more than the last-level cache holds
+            lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 30), 5, 30)))
+            del other
+            torch.cuda.empty_cache()
+        result["configs"] = lines
+
+    result["roofline"]["device_copy_GBps"] = round(_device_copy_gbps(dev, stream), 1)
+    if not a.no_cpu_baseline:
+        # a bounded sample: the first sequences of pool 0, copied to the host
+        nsamp = min(wl0.batch, 16)
+        result["cpu_baseline"] = _cpu_baseline(wl0.to("cpu"), nsamp, wl0.batch)
+    print(json.dumps(result, ensure_ascii=False))
+    return 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the read-only probe of c2's gather pattern
+# ---------------------------------------------------------------------------------------------------------------
+def _bench_probe_gather(a) -> int:
+    """Reads exactly the pages c2's partition kernel reads, in the same order and grouping (one workgroup of four
+    waves per (sequence, kv head), each wave every fourth 64-token step, 16 bytes per lane, non-temporal), and does
+    no arithmetic: what the memory system gives this access pattern."""
+    import torch
+
+    from triton_op_amd import _cabi
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    lib = _cabi.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream(dev)
+    sh = C.c_void_p(stream.cuda_stream)
+    cfg = _Config("c2", dev, a.pools, a.partition_size, a.batch or None)
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+
+    def call(i):
+        rc = lib.pa_debug_gather_probe(C.byref(cfg.plans[i % len(cfg.plans)].args), C.c_void_p(sink.data_ptr()), sh)
+        if rc:
+            _cabi.check(rc, "pa_debug_gather_probe")
+
+    for i in range(SETTLE_CALLS):
+        call(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(a.steps):
+        call(i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / a.steps
+    gbps = cfg.kv_bytes / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "read-only gather probe of c2's page pattern (no arithmetic)", "value": round(gbps, 1), "unit": "GB/s",
+        "us_per_call": round(us, 2), "n_gpus": 1, "steps": a.steps, "warmup": SETTLE_CALLS, "ms_per_step": round(us / 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "probe_gather_" + cfg.wl0.name, "bytes_per_call": cfg.kv_bytes,
+                   "kv_pools_rotated": len(cfg.plans)},
+        "roofline": {"bound": "hbm", "kernel": "pa_gather_probe_kernel", "achieved": round(gbps, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+    }, ensure_ascii=False))
+    return 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the KV-cache write kernels
+# ---------------------------------------------------------------------------------------------------------------
 def _bench_kv_cache(a) -> int:
     """The step before the decode path: `kv_write` appends 64 prompts of 4096 tokens (8 kv heads, head 128, bf16
     rows) to an FP8 paged cache with per-token scales in one call; `kv_quantize` converts the c2 cache pool
     (20480 pages of 16 tokens) from bf16 to FP8 with per-token scales.  Bytes counted: rows or cache read once,
-    cache and scales written once."""
+    cache and scales written once.  These kernels read and write in about equal parts, and a plain device copy
+    (hipMemcpyDtoD, the same mix) is the bound they are held against: `roofline.peak` stays the published 8 TB/s,
+    `roofline.frac_of_device_copy` is the fraction of the copy rate measured in the same process."""
     import torch
 
     import triton_op_amd as T
@@ -149,6 +552,7 @@ def _bench_kv_cache(a) -> int:
     us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
     us_median = us[len(us) // 2]
     achieved = nbytes / (us_median * 1e-6) / 1e9
+    copy_gbps = _device_copy_gbps(dev, stream)
     result = {
         "metric": "KV-cache write GB/s (rows read + FP8 cache and scales written)", "value": round(achieved, 1),
         "unit": "GB/s", "us_per_call": round(us_median, 2), "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -156,7 +560,10 @@ def _bench_kv_cache(a) -> int:
         "dtype": "bf16 in, fp8_e4m3fn + f32 scales out", "data": "synthetic",
         "config": {"workload": name, "kv_heads": h, "head_size": d, "block_size": bs, "bytes_per_call": nbytes},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "device_copy_GBps": round(copy_gbps, 1), "frac_of_device_copy": round(achieved / copy_gbps, 4),
+                     "bound_note": "mixed read/write stream: the measured rate of a plain device copy (read + write "
+                                   "bytes) is the practical bound, the published peak is a read-stream figure"},
     }
     if not a.no_cpu_baseline:
         cpu_sample()  # warm-up
@@ -176,180 +583,22 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2")
+    ap.add_argument("--workload", default="", help="default: c2 as the headline plus c2@256, c3, c4, c5 in `configs`")
     ap.add_argument("--partition-size", type=int, default=0, help="0 = let the tuning layer choose")
     ap.add_argument("--pools", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="default run: the headline only")
     ap.add_argument("--batch", type=int, default=0, help="override the batch size (debugging only)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op shards by kv head or "
               "by sequence with no exchange); run with --gpus 1", file=sys.stderr)
         return 2
-
     if a.workload in ("kv_write", "kv_quantize"):
         return _bench_kv_cache(a)
-
-    import torch
-
-    import triton_op_amd as T
-    from triton_op_amd import _cabi
-    from triton_op_amd import workloads as W
-
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        return 2
-    lib = _cabi.load_library()
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    props = torch.cuda.get_device_properties(dev)
-
-    # ---- workload: `pools` independent copies (different seeds) ----------------------------------------
-    plans, wls = [], []
-    for i in range(a.pools):
-        wl = W.make_config(a.workload, device=dev, batch=a.batch or None)
-        if i:
-            # same shapes, different page contents and block tables
-            cfg = dict(name=wl.name, seed=wl.meta["seed"] + 100 * i, batch=wl.batch, num_q_heads=wl.num_q_heads,
-                       num_kv_heads=wl.num_kv_heads, block_size=wl.block_size, context_lens=wl.context_lens.cpu(),
-                       q_len=wl.q_len, q_lens=None if wl.q_lens is None else wl.q_lens.cpu(),
-                       kv_dtype=wl.meta["kv_dtype"], scale_mode=wl.meta["scale_mode"], device=dev)
-            wl = W.make_decode_workload(**cfg)
-        out = torch.empty_like(wl.query)
-        ps = a.partition_size or None
-        plan = T.plan_decode(out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
-                             wl.softmax_scale, wl.q_len, wl.max_context_len, torch.bfloat16, None, wl.key_scale,
-                             wl.value_scale, partition_size=ps, query_lens=wl.q_lens)
-        plans.append(plan)
-        wls.append(wl)
-    wl0 = wls[0]
-    _FULL_BATCH[0] = wl0.batch
-    kv_bytes = wl0.kv_bytes()
-    stream = torch.cuda.current_stream(dev)
-    sh = C.c_void_p(stream.cuda_stream)
-    n = len(plans)
-
-    def step(i):
-        p = plans[i % n]
-        rc = lib.pa_decode(C.byref(p.args), sh)
-        if rc:
-            _cabi.check(rc, "pa_decode")
-
-    # ---- whole-op timing ---------------------------------------------------------------------------------
-    for i in range(a.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        step(i)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
-
-    # per-call device time from events on the launch stream (median is the headline µs/call)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-    for i in range(a.steps):
-        evs[i][0].record(stream)
-        step(i)
-        evs[i][1].record(stream)
-    torch.cuda.synchronize()
-    call_us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
-    us_median = call_us[len(call_us) // 2]
-    us_mean = sum(call_us) / len(call_us)
-
-    # ---- the dominant kernel alone (roofline) --------------------------------------------------------------
-    # Its average duration from HIP events on the launch stream.  When the partition kernel is the whole call
-    # (one partition per sequence: c2), one event pair brackets the region of `steps`
-    # back-to-back launches, which is what a kernel trace's average sees; otherwise other kernels run in
-    # between and every launch gets an event pair of its own (which also brackets its dispatch).
-    solo = plans[0].args.max_num_partitions == 1
-    if solo:
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for i in range(a.steps):
-            rc = lib.pa_decode_partition(C.byref(plans[i % n].args), sh)
-            if rc:
-                _cabi.check(rc, "pa_decode_partition")
-        e1.record(stream)
-        torch.cuda.synchronize()
-        k_us_avg = e0.elapsed_time(e1) * 1e3 / a.steps
-        k_timing = f"one event pair around {a.steps} back-to-back launches"
-    else:
-        kevs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-        for i in range(a.steps):
-            p = plans[i % n]
-            kevs[i][0].record(stream)
-            rc = lib.pa_decode_partition(C.byref(p.args), sh)
-            kevs[i][1].record(stream)
-            if rc:
-                _cabi.check(rc, "pa_decode_partition")
-            if p.args.max_num_partitions > 1:
-                lib.pa_decode_reduce(C.byref(p.args), sh)
-        torch.cuda.synchronize()
-        k_us = [e0.elapsed_time(e1) * 1e3 for e0, e1 in kevs]
-        k_us_avg = sum(k_us) / len(k_us)
-        k_timing = "an event pair around every launch (planning kernel included when the launch uses one)"
-    achieved = kv_bytes / (k_us_avg * 1e-6) / 1e9
-
-    # ---- a plain device copy, for scale -------------------------------------------------------------------
-    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-    dst = torch.empty_like(src)
-    for _ in range(3):
-        dst.copy_(src)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(10):
-        dst.copy_(src)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    copy_gbps = 10 * 2 * (1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9
-    del src, dst
-
-    traffic = HBM_TRAFFIC_BYTES.get((wl0.name, int(plans[0].args.partition_size)))
-
-    result = {
-        "metric": METRIC,
-        "value": round(kv_bytes / (us_median * 1e-6) / 1e9, 1),
-        "unit": "GB/s (KV bytes / median µs per call)",
-        "us_per_call": round(us_median, 2),
-        "us_per_call_mean": round(us_mean, 2),
-        "pct_of_hbm_peak": round(kv_bytes / (us_median * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100, 2),
-        "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
-        "ms_per_step": round(wall_ms, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "fp8_e4m3fn KV on FP8 MFMA (bf16 Q and P carried as two FP8 terms), f32 accumulate and softmax, bf16 out",
-        "data": "synthetic",
-        "config": {
-            "workload": wl0.name,
-            "batch": wl0.batch, "q_heads": wl0.num_q_heads, "kv_heads": wl0.num_kv_heads,
-            "head_size": wl0.head_size, "q_len": wl0.q_len, "block_size": wl0.block_size,
-            "context_len_max": wl0.max_context_len, "partition_size": int(plans[0].args.partition_size),
-            "kv_bytes_per_call": kv_bytes, "kv_pools_rotated": n, "device": props.name,
-            "compute_units": props.multi_processor_count,
-        },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": _partition_kernel_name(wl0),
-            "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": traffic,
-            "kernel_us_avg": round(k_us_avg, 2),
-            "kernel_timing": k_timing,
-            "algorithmic_bytes_per_launch": kv_bytes,
-            "device_copy_GBps": round(copy_gbps, 1),
-        },
-    }
-    if not a.no_cpu_baseline:
-        # a bounded sample: the first sequences of pool 0, copied to the host
-        nsamp = min(wl0.batch, 16)
-        result["cpu_baseline"] = _cpu_baseline(wl0.to("cpu"), nsamp)
-    print(json.dumps(result, ensure_ascii=False))
-    return 0
+    if a.workload == "probe_gather":
+        return _bench_probe_gather(a)
+    return _bench_decode(a)
 
 
 if __name__ == "__main__":

@@ -95,7 +95,9 @@ typedef struct PaDecodeArgs {
   const float* query_scale;   /* optional; per tensor: 1 value, per token: [B, Hkv*Ge, 1] */
   const float* key_scale;     /* optional */
   const float* value_scale;   /* optional */
-  const float* alibi_slopes;  /* optional, [Hkv*G] */
+  const float* alibi_slopes;  /* optional, [Hkv*G]: one slope per query HEAD, shared by the q new tokens of a head (the
+                                 reference kernel indexes [Hkv*q*G] like sinks, pa_decode_triton_gluon_fp8.py:323-327;
+                                 the two agree for q_len == 1) */
   const float* sinks;         /* optional, [Hkv*Ge]: attention-sink logit of every query row (natural-log domain) */
   float* exp_sums;
   float* max_logits;
@@ -108,7 +110,9 @@ typedef struct PaDecodeArgs {
   int32_t q_len;               /* q (the maximum over the batch when q_lens is given) */
   int32_t head_size;           /* D, 128 */
   int32_t block_size;          /* 16, 64 or 1024 */
-  int32_t max_num_partitions;  /* P: partition axis length of the three buffers */
+  int32_t max_num_partitions;  /* P: partition axis length of the three buffers; P * partition_size must cover the
+                                  longest context_len (the caller's max_sequence_length sizes it): tokens beyond it
+                                  are not attended to, whatever P is */
   int32_t partition_size;      /* tokens per partition, a multiple of 256 */
   int32_t query_dtype;         /* PA_DTYPE_* */
   int32_t kv_dtype;            /* PA_DTYPE_* */
@@ -173,6 +177,24 @@ int pa_decode_reduce(const PaDecodeArgs* args, void* hip_stream);
 /* Both stages back to back on one stream: the body of the reference's paged_attention_decode.  Stage 2
  * skips the sequences stage 1 has finished, and is not launched when max_num_partitions == 1 (no sinks). */
 int pa_decode(const PaDecodeArgs* args, void* hip_stream);
+
+/*
+ * What the launch layer would do with these arguments, as text: the partition kernel's instantiation, its grid
+ * and where its workgroups take their items from, e.g.
+ *   "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
+ *   "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 6512, sorted items".
+ * The choice is a function of the arguments and the device's CU count alone.  (The reference's counterpart is
+ * the kernel selection in pa_decode_triton_gluon_fp8.py:1492-1509.)  Launches nothing.
+ *
+ * Limits of the two launch modes that need a workspace (beyond them the call is launched in plain order, with
+ * the same results): the queued launch of ragged batches holds its item table in LDS and takes at most 2048
+ * sequences; the sorted dispatch's planning kernel takes at most 4096.
+ *
+ * Environment: none of the library's behaviour depends on environment variables unless the process was started
+ * with PA_DECODE_DEBUG=1, which enables the tuning switches PA_DECODE_WAVES, PA_DECODE_QUEUE, PA_DECODE_SHARED
+ * and PA_DECODE_SORTED (read once, at the first launch).
+ */
+int pa_decode_launch_info(const PaDecodeArgs* args, char* text, int32_t text_bytes);
 
 /*
  * pa_decode for callers that cannot allocate device memory and have no partition buffers to pass: code under
@@ -245,6 +267,15 @@ int pa_quantize_kv_cache(const void* key_cache_bf16, const void* value_cache_bf1
  * with the format definition code by code.
  */
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream);
+
+/*
+ * Measurement hook: a read-only probe of the memory access pattern of stage 1.  For the same arguments it reads
+ * the K and V bytes that the partition kernel for up to 16 query rows reads (FP8 cache, block size 16, dense
+ * layout; anything else is PA_ERR_UNSUPPORTED), with the same workgroup decomposition, load width and cache
+ * policy, and does no arithmetic: its duration is what the memory system gives the gather pattern.  sink: at
+ * least 64 int32 of device memory (written only in a case that does not occur; it keeps the loads alive).
+ */
+int pa_debug_gather_probe(const PaDecodeArgs* args, int32_t* sink, void* hip_stream);
 
 #ifdef __cplusplus
 }

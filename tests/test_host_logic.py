@@ -145,6 +145,40 @@ def test_entry_point_rejects_group_and_block_size():
                       torch.zeros(1, 4, dtype=torch.int32), 0.1, 1, 40)
 
 
+def test_kv_cache_writers_reject_tensors_on_another_device(monkeypatch):
+    """Every tensor handed to the cache writers is dereferenced on the GPU: one that lives elsewhere (a
+    slot_mapping built on the host, a CPU scale tensor) must raise before anything is launched.  The check is
+    reached on this GPU-less machine by presenting the key rows as a tensor of another device type."""
+    from triton_op_amd import kv_cache as KC
+
+    class _Launched(Exception):
+        pass
+
+    def _no_launch():
+        raise _Launched("the library must not be reached")
+
+    monkeypatch.setattr(KC._cabi, "load_library", _no_launch)
+    t, h, d, bs, nblk = 32, 2, 128, 16, 4
+    key = torch.zeros(t, h, d, dtype=torch.bfloat16, device="meta")
+    value = torch.zeros(t, h, d, dtype=torch.bfloat16, device="meta")
+    kc = torch.zeros(nblk, h, d // 16, bs, 16, dtype=torch.float8_e4m3fn, device="meta")
+    vc = torch.zeros(nblk, h, d, bs, dtype=torch.float8_e4m3fn, device="meta")
+    ks = torch.zeros(nblk, h, bs, 1, device="meta")
+    vs = torch.zeros(nblk, h, bs, 1, device="meta")
+    slots = torch.zeros(t, dtype=torch.int64, device="meta")
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: self.device.type in ("cuda", "meta")))
+    good = dict(key=key, value=value, key_cache=kc, value_cache=vc, slot_mapping=slots, key_scale=ks, value_scale=vs)
+    for name in ("value", "key_cache", "value_cache", "slot_mapping", "key_scale", "value_scale"):
+        bad = dict(good)
+        bad[name] = torch.zeros(good[name].shape, dtype=good[name].dtype)  # the same tensor on the CPU
+        with pytest.raises(ValueError, match=f"{name} is on cpu"):
+            KC.kv_cache_write(**bad)
+    kc16 = torch.zeros(nblk, h, d // 8, bs, 8, dtype=torch.bfloat16, device="meta")
+    vc16 = torch.zeros(nblk, h, d, bs, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="value_cache is on cpu"):
+        KC.quantize_kv_cache_symmetric(kc16, vc16)
+
+
 def test_library_path_must_exist(monkeypatch):
     monkeypatch.setattr(_cabi, "_lib", None)
     with pytest.raises(_cabi.PaDecodeLibraryError, match="is missing"):

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = [os.path.join(HERE, "csrc", "pa_decode.hip"), os.path.join(HERE, "csrc", "pa_kv_cache.hip")]
 HEADERS = [os.path.join(HERE, "..", "include", "pa_decode.h")] + [
     os.path.join(HERE, "csrc", h)
-    for h in ("pa_common.h", "pa_partition_kernel.h", "pa_partition_shared_kernel.h", "pa_plan_kernel.h",
+    for h in ("pa_common.h", "pa_partition_kernel.h", "pa_partition_shared_kernel.h", "pa_plan_kernel.h", "pa_probe_kernel.h",
               "pa_reduce_kernel.h")]
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 

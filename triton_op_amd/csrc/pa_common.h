@@ -190,11 +190,15 @@ __device__ __forceinline__ void zero_output_rows(const PaDecodeArgs& a, int b, i
 // They are non-temporal (the cache is streamed once).
 // The loads count in vmcnt like any other vector load, but the compiler does not see them: whoever reads
 // the LDS bytes waits with dma_wait<N>() (at most N vector memory operations still outstanding) first.
+// M0 carries the LDS address and is named as clobbered, so the compiler keeps no value of its own in it across
+// the statement (it reserves M0 and warns about any clobber that names it; that is what is wanted here).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma_load16(const void* gptr, uint32_t lds_offset) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory", "m0");
 }
 __device__ __forceinline__ void dma_load4(const void* gptr, uint32_t lds_offset) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory", "m0");
 }
 // the same with the address split into a wave-uniform base and a 32-bit per-lane byte offset; STREAM = false
 // for bytes whose 128-byte lines other loads will touch again soon (those must stay in L2)
@@ -210,12 +214,13 @@ __device__ __forceinline__ void dma_load16(const void* base, uint32_t lane_offse
   if constexpr (STREAM)
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" ::"v"(lane_offset), "s"(sb),
                  "s"(lds_offset)
-                 : "memory");
+                 : "memory", "m0");
   else
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(sb),
                  "s"(lds_offset)
-                 : "memory");
+                 : "memory", "m0");
 }
+#pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void dma_wait() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

@@ -10,6 +10,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 #include <stdlib.h>
 
 #include <mutex>
@@ -19,6 +20,7 @@
 #include "pa_partition_kernel.h"
 #include "pa_partition_shared_kernel.h"
 #include "pa_plan_kernel.h"
+#include "pa_probe_kernel.h"
 #include "pa_reduce_kernel.h"
 
 // Scratch of pa_decode_noalloc, the entry point for callers that can neither allocate nor pass partition buffers:
@@ -47,8 +49,6 @@ __global__ void pa_fp8_decode_kernel(const uint8_t* codes, float* out, int n) {
 }
 
 thread_local int g_last_hip_error = 0;
-// set by the partition stage's launch: did it go through the planning kernel's lists (sorted dispatch)?
-thread_local bool g_used_item_lists = false;
 
 int check_common(const PaDecodeArgs* a) {
   if (!a) return PA_ERR_NULL_POINTER;
@@ -75,18 +75,20 @@ int device_num_cus() {
   return n;
 }
 
-// The queued launch is used when the caller gave a workspace and per-sequence query lengths and a kv head has
-// more than one 16-row query tile (tiles of padding rows only are then common): a resident grid pulls live
-// items from a counter.  Otherwise the only workgroups with nothing to do are partitions past a sequence's end,
-// which the plain launch orders last; there the queue's bookkeeping costs more than it saves (measured: +10 %
-// on a uniform batch).
-bool use_queue(const PaDecodeArgs& a) {
-  static const bool off = [] {
-    const char* e = getenv("PA_DECODE_QUEUE");
-    return e && e[0] == '0';
+// Experiment switches.  They exist for tuning runs only and are dead unless the process was started with
+// PA_DECODE_DEBUG=1, so a serving process's launches never depend on stray environment variables:
+//   PA_DECODE_WAVES=n    waves per workgroup of pa_partition_kernel
+//   PA_DECODE_QUEUE=0    no queued launch          PA_DECODE_SHARED=0   one workgroup per 16-row tile, always
+//   PA_DECODE_SORTED=0|1 never / always the sorted dispatch (when the workspace has room)
+// All are read once, at the first launch.
+int debug_switch(const char* name, int unset) {
+  static const bool enabled = [] {
+    const char* e = getenv("PA_DECODE_DEBUG");
+    return e && e[0] == '1';
   }();
-  return !off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr &&
-         a.q_len * a.group_size > 16;
+  if (!enabled) return unset;
+  const char* e = getenv(name);
+  return e ? atoi(e) : unset;
 }
 
 // Bytes of workspace the sorted dispatch needs: the header and one (sequence, partition) pair per possible item.
@@ -98,153 +100,213 @@ long long full_workspace_bytes(int num_seqs, int max_num_partitions) {
   return plan_workspace_bytes(num_seqs, max_num_partitions) + 4LL * num_seqs;
 }
 
-// The sorted dispatch pays a small extra kernel, and ordering only matters when workgroups are handed out in
-// several rounds: it is used when the launch has more than twice as many workgroups as the GPU holds at once
-// and the caller's workspace has room for the list.  PA_DECODE_SORTED=0 switches it off, =1 drops the size rule.
-bool use_sorted_items(const PaDecodeArgs& a, long long blocks, int workgroups_per_cu) {
-  static const int mode = [] {
-    const char* e = getenv("PA_DECODE_SORTED");
-    return e ? atoi(e) : -1;
-  }();
-  if (mode == 0 || a.workspace == nullptr || a.num_seqs > kPlanMaxSeqs) return false;
-  if (a.workspace_bytes < plan_workspace_bytes(a.num_seqs, a.max_num_partitions)) return false;
-  return mode == 1 || blocks > 2LL * device_num_cus() * workgroups_per_cu;
+// pa_partition_kernel, waves per workgroup: 128 tokens (2 steps) per wave at least, and at most 4 waves (the
+// merge buffer of a workgroup is WAVES * 8 KiB of LDS).  Eight waves (one partition where four waves take two)
+// were measured and lose: a wave's chain of 1.4 us steps is what a small batch waits for, and more partitions
+// shorten it where more waves per workgroup cannot go below the second kernel's cost anyway.
+int waves_for_partition_size(int partition_size) { return partition_size >= 512 ? 4 : 2; }
+
+// More than one 16-row query tile per kv head over an FP8 cache: the tiles share one pass over the pages
+// (pa_partition_shared_kernel).
+bool use_shared_stream(int kv_dtype, int rows_per_group) {
+  static const bool off = debug_switch("PA_DECODE_SHARED", 1) == 0;
+  return !off && kv_dtype == PA_DTYPE_FP8_E4M3FN && rows_per_group > 16;
+}
+
+// Everything the launch layer decides for one call, from the arguments alone (pure host arithmetic): which
+// partition kernel in which instantiation, how many workgroups, and how they get their items.
+struct LaunchChoice {
+  bool shared;      // pa_partition_shared_kernel (else pa_partition_kernel, one workgroup per 16-row tile)
+  bool fp8;         // FP8 cache (else bf16)
+  bool per_token;   // per-token kv scales
+  bool bs16;        // constant in-page strides: block size 16 with the default dense layout
+  int waves;        // waves per workgroup
+  int per_cu;       // workgroups of this instantiation that fit a CU
+  bool queue;       // a resident grid pulls live items from a counter in the workspace
+  bool sorted;      // items come from the planning kernel's list in the workspace
+  bool listed_reduce;  // ... and pa_decode's reduce stage walks the planning kernel's list of multi-partition sequences
+  long long blocks; // workgroups launched
+};
+
+LaunchChoice choose_launch(const PaDecodeArgs& a) {
+  LaunchChoice c{};
+  const int ge = a.q_len * a.group_size;
+  c.fp8 = a.kv_dtype == PA_DTYPE_FP8_E4M3FN;
+  c.per_token = a.kv_quant_mode == PA_QUANT_PER_TOKEN;
+  c.bs16 = c.fp8 && a.block_size == 16 && a.stride_k_c == 256 &&
+           (a.v_transposed ? a.stride_v_2 == 2048 : a.stride_v_2 == 16);
+  c.shared = use_shared_stream(a.kv_dtype, ge);
+  long long items;  // (sequence, partition) pairs times kv heads times row tiles
+  if (c.shared) {
+    // ring depth / waves per SIMD: without per-token scales the kernel fits 128 registers, and a fourth
+    // workgroup per CU is worth more than a deeper ring (measured); with them it needs about 140
+    c.waves = 4;
+    c.per_cu = c.per_token ? 3 : 4;
+    items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
+  } else {
+    // no more waves than it takes to fill the GPU's wave slots (8 per CU): with 8 workgroups or more per CU one
+    // wave each is best (no merge, more independent streams: 256 sequences x 8 kv heads x 512 tokens 57.7 ->
+    // 44.8 us), with 4 per CU two.  But a wave keeps at most 16 steps (1024 tokens) to itself, or the longest
+    // items of a ragged batch finish the launch alone, one slow wave each (256 sequences of 1..4096 tokens:
+    // 196 us with one wave per workgroup against 179 us with four).
+    static const int forced = debug_switch("PA_DECODE_WAVES", 0);
+    items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * ((ge + 15) / 16);
+    int w = waves_for_partition_size(a.partition_size);
+    if (forced > 0) {
+      w = forced;
+    } else {
+      const long long slots = 8LL * device_num_cus();
+      int need = 1;  // waves per workgroup that fill the slots, or keep a wave's share at 1024 tokens
+      while (need < w && (items * need < slots || a.partition_size > 1024 * need)) need *= 2;
+      w = need;
+    }
+    c.waves = w >= 4 ? 4 : (w >= 2 ? 2 : 1);
+    c.per_cu = 8 / c.waves;
+  }
+  c.blocks = items;
+  // The queued launch is used when the caller gave a workspace and per-sequence query lengths and a kv head has
+  // more than one 16-row query tile (tiles of padding rows only are then common): a resident grid pulls live
+  // items from a counter.  Otherwise the only workgroups with nothing to do are partitions past a sequence's
+  // end, which the plain launch orders last; there the queue's bookkeeping costs more than it saves (measured:
+  // +10 % on a uniform batch).  Batches of more than kQueueMaxSeqs sequences (the item table in LDS) are
+  // launched plainly.
+  static const bool queue_off = debug_switch("PA_DECODE_QUEUE", 1) == 0;
+  c.queue = !c.shared && !queue_off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr &&
+            ge > 16;
+  if (c.queue) {
+    const long long resident = (long long)device_num_cus() * c.per_cu;
+    c.blocks = resident < items ? resident : items;
+  }
+  // The sorted dispatch pays a small extra kernel, and ordering only matters when workgroups are handed out in
+  // several rounds: it is used when the launch has more than twice as many workgroups as the GPU holds at once
+  // and the caller's workspace has room for the list (batches of more than kPlanMaxSeqs sequences, the planning
+  // kernel's LDS tables, are launched in plain order).
+  static const int sorted_mode = debug_switch("PA_DECODE_SORTED", -1);
+  c.sorted = !c.queue && sorted_mode != 0 && a.workspace != nullptr && a.num_seqs <= kPlanMaxSeqs &&
+             a.workspace_bytes >= plan_workspace_bytes(a.num_seqs, a.max_num_partitions) &&
+             (sorted_mode == 1 || items > 2LL * device_num_cus() * c.per_cu);
+  c.listed_reduce = c.sorted && !a.sinks &&
+                    a.workspace_bytes >= full_workspace_bytes(a.num_seqs, a.max_num_partitions);
+  return c;
+}
+
+int launch_status() {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return PA_OK;
+  g_last_hip_error = (int)e;
+  return PA_ERR_LAUNCH;
 }
 
 int launch_plan(const PaDecodeArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(pa_plan_kernel, dim3(1), dim3(1024), 0, stream, a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
+  return launch_status();
 }
-
-template <int NT, int KVT, bool PT, bool BS16, int W>
-int launch_partition_w(const PaDecodeArgs& a, hipStream_t stream) {
-  constexpr int OCC = NT == 1 ? 2 : 1;
-  const int ge = a.q_len * a.group_size;
-  const int row_tiles = (ge + 16 * NT - 1) / (16 * NT);
-  const long long blocks = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * row_tiles;
-  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  if (use_queue(a)) {
-    long long resident = (long long)device_num_cus() * 4 * OCC / W;
-    resident = resident < blocks ? resident : blocks;
-    PaDecodeArgs k = a;
-    k.flags = 0;
-    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)resident),
-                       dim3(64 * W), 0, stream, k);
-  } else {
-    PaDecodeArgs k = a;
-    k.flags = 0;
-    if (use_sorted_items(a, blocks, 4 * OCC / W)) {
-      if (!(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST)) {
-        const int rc = launch_plan(a, stream);
-        if (rc) return rc;
-      }
-      k.flags = kFlagSortedItems;
-      g_used_item_lists = true;
-    }
-    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)blocks), dim3(64 * W), 0,
-                       stream, k);
-  }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
-}
-
 
 // pa_partition_kernel is instantiated with one 16-row query tile per workgroup (NT = 1): a bf16 cache with
 // more than 16 query rows per kv head gets one workgroup per tile (they read the same pages at the same time
-// from the same L2, and tiles that hold only padding rows cost nothing); an FP8 cache goes to
-// pa_partition_shared_kernel.
-// Waves per workgroup: 128 tokens (2 steps) per wave at least, and at most 4 waves (the merge buffer of a
-// workgroup is WAVES * 8 KiB of LDS).  Eight waves (one partition where four waves take two) were
-// measured and lose: a wave's chain of 1.4 us steps is what a small batch waits for, and more partitions
-// shorten it where more waves per workgroup cannot go below the second kernel's cost anyway.
-int waves_for_partition_size(int partition_size) { return partition_size >= 512 ? 4 : 2; }
-// ... and no more waves than it takes to fill the GPU's wave slots (8 per CU): with 8 workgroups or more per CU
-// one wave each is best (no merge, more independent streams: 256 sequences x 8 kv heads x 512 tokens 57.7 -> 44.8
-// us), with 4 per CU two.  But a wave keeps at most 16 steps (1024 tokens) to itself, or the longest items of a
-// ragged batch finish the launch alone, one slow wave each (256 sequences of 1..4096 tokens: 196 us with one
-// wave per workgroup against 179 us with four).
-int waves_per_workgroup(const PaDecodeArgs& a) {
-  static const int forced = [] {
-    const char* e = getenv("PA_DECODE_WAVES");
-    return e ? atoi(e) : 0;
-  }();
-  int w = waves_for_partition_size(a.partition_size);
-  if (forced > 0) {
-    w = forced;
-  } else {
-    const long long workgroups = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions *
-                                 ((a.q_len * a.group_size + 15) / 16);
-    const long long slots = 8LL * device_num_cus();
-    int need = 1;  // waves per workgroup that fill the slots, or keep a wave's share at 1024 tokens
-    while (need < w && (workgroups * need < slots || a.partition_size > 1024 * need)) need *= 2;
-    w = need;
-  }
-  return w >= 4 ? 4 : (w >= 2 ? 2 : 1);
+// from the same L2, and tiles that hold only padding rows cost nothing).
+template <int KVT, bool PT, bool BS16, int W>
+void launch_partition_w(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+  constexpr int OCC = 2;
+  if (c.queue)
+    hipLaunchKernelGGL((pa_partition_kernel<1, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
+                       stream, k);
+  else
+    hipLaunchKernelGGL((pa_partition_kernel<1, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
+                       stream, k);
 }
 
-// More than one 16-row query tile per kv head over an FP8 cache: the tiles share one pass over the pages
-// (pa_partition_shared_kernel).  PA_DECODE_SHARED=0 falls back to one workgroup per tile.
-bool use_shared_stream(int kv_dtype, int rows_per_group) {
-  static const bool off = [] {
-    const char* e = getenv("PA_DECODE_SHARED");
-    return e && e[0] == '0';
-  }();
-  return !off && kv_dtype == PA_DTYPE_FP8_E4M3FN && rows_per_group > 16;
+template <int KVT, bool PT, bool BS16>
+void launch_partition_tile(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+  if (c.waves == 4) return launch_partition_w<KVT, PT, BS16, 4>(k, c, stream);
+  if (c.waves == 2) return launch_partition_w<KVT, PT, BS16, 2>(k, c, stream);
+  return launch_partition_w<KVT, PT, BS16, 1>(k, c, stream);
 }
 
 template <bool PT, bool BS16>
-int launch_partition_shared(const PaDecodeArgs& a, hipStream_t stream) {
-  const long long blocks = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
-  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  // ring depth / waves per SIMD: without per-token scales the kernel fits 128 registers, and a fourth workgroup
-  // per CU is worth more than a deeper ring (measured); with them it needs about 140
-  constexpr int kWorkgroupsPerCu = PT ? 3 : 4;
+void launch_partition_shared(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+  if constexpr (PT)
+    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)c.blocks), dim3(256), 0, stream, k);
+  else
+    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)c.blocks), dim3(256), 0, stream, k);
+}
+
+// stage 1 as chosen: the planning kernel when the items are to be sorted, then the partition kernel
+int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t stream) {
+  if (c.blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
   PaDecodeArgs k = a;
   k.flags = 0;
-  if (use_sorted_items(a, blocks, kWorkgroupsPerCu)) {
+  if (c.sorted) {
     if (!(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST)) {
       const int rc = launch_plan(a, stream);
       if (rc) return rc;
     }
     k.flags = kFlagSortedItems;
-    g_used_item_lists = true;
   }
-  if constexpr (PT)
-    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, k);
-  else
-    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, k);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
+  if (!c.fp8) {
+    launch_partition_tile<PA_DTYPE_BF16, false, false>(k, c, stream);
+  } else if (c.shared) {
+    if (c.bs16)
+      c.per_token ? launch_partition_shared<true, true>(k, c, stream) : launch_partition_shared<false, true>(k, c, stream);
+    else
+      c.per_token ? launch_partition_shared<true, false>(k, c, stream) : launch_partition_shared<false, false>(k, c, stream);
+  } else if (c.bs16) {
+    c.per_token ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, true>(k, c, stream)
+                : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, true>(k, c, stream);
+  } else {
+    c.per_token ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, false>(k, c, stream)
+                : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, false>(k, c, stream);
   }
+  return launch_status();
+}
+
+// the argument checks of stage 1
+int check_partition(const PaDecodeArgs* a) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!a->query || !a->key_cache || !a->value_cache || !a->block_tables) return PA_ERR_NULL_POINTER;
+  if (a->block_size != 16 && a->block_size != 64 && a->block_size != 1024) return PA_ERR_UNSUPPORTED;
+  if (a->kv_dtype != PA_DTYPE_BF16 && a->kv_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
+  if (a->query_dtype != PA_DTYPE_BF16 && a->query_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
+  if (a->kv_quant_mode != PA_QUANT_NONE && (!a->key_scale || !a->value_scale)) return PA_ERR_NULL_POINTER;
+  if (a->query_quant_mode != PA_QUANT_NONE && !a->query_scale) return PA_ERR_NULL_POINTER;
+  if (a->kv_quant_mode < -1 || a->kv_quant_mode > 1 || a->query_quant_mode < -1 || a->query_quant_mode > 1)
+    return PA_ERR_UNSUPPORTED;
+  if (a->kv_quant_mode == PA_QUANT_PER_TOKEN && a->kv_dtype != PA_DTYPE_FP8_E4M3FN)
+    return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
+  const int esz = a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
+  // 16-byte vector loads: every stride that moves a vector must keep it 16-byte aligned
+  if ((a->stride_k_b * esz) % 16 || (a->stride_k_h * esz) % 16 || (a->stride_k_c * esz) % 16 ||
+      (a->stride_v_b * esz) % 16 || (a->stride_v_h * esz) % 16 || (a->stride_v_2 * esz) % 16)
+    return PA_ERR_BAD_SHAPE;
+  const int qsz = a->query_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
+  if ((a->stride_q_s * qsz) % 16 || (a->stride_q_h * qsz) % 16) return PA_ERR_BAD_SHAPE;
+  if ((a->stride_tmp_g * 2) % 16 || (a->stride_tmp_p * 2) % 16 || (a->stride_tmp_h * 2) % 16 || (a->stride_tmp_s * 2) % 16 ||
+      (reinterpret_cast<uintptr_t>(a->tmp_output) & 15))
+    return PA_ERR_BAD_SHAPE;
+  if (a->kv_quant_mode == PA_QUANT_PER_TOKEN && (a->stride_kvscale_b % 4 || a->stride_kvscale_h % 4))
+    return PA_ERR_BAD_SHAPE;
+  if ((long long)(4 * 3 + 3) * a->stride_k_c * esz + 15 * 16 >= (1LL << 32)) return PA_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(a->key_cache) | reinterpret_cast<uintptr_t>(a->value_cache) |
+       reinterpret_cast<uintptr_t>(a->query)) & 15)
+    return PA_ERR_BAD_SHAPE;
   return PA_OK;
 }
 
-template <int KVT, bool PT, bool BS16>
-int launch_partition_tile(const PaDecodeArgs& a, hipStream_t stream) {
-  const int w = waves_per_workgroup(a);
-  if (w == 4) return launch_partition_w<1, KVT, PT, BS16, 4>(a, stream);
-  if (w == 2) return launch_partition_w<1, KVT, PT, BS16, 2>(a, stream);
-  return launch_partition_w<1, KVT, PT, BS16, 1>(a, stream);
-}
-
-int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
+// ... and of stage 2
+int check_reduce(const PaDecodeArgs* a) {
   int rc = check_common(a);
   if (rc) return rc;
   if (!a->output) return PA_ERR_NULL_POINTER;
   if (a->stride_out_h % 2 || a->stride_out_s % 2 || a->stride_tmp_g % 2 || a->stride_tmp_p % 2 ||
       a->stride_tmp_h % 2 || a->stride_tmp_s % 2)
     return PA_ERR_BAD_SHAPE;
+  return PA_OK;
+}
+
+int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
+  int rc = check_reduce(a);
+  if (rc) return rc;
   const long long blocks = (long long)a->num_seqs * a->num_kv_heads * ((a->q_len * a->group_size + 15) / 16);
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
@@ -386,71 +448,41 @@ int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int3
 }
 
 int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
-  int rc = check_common(a);
+  const int rc = check_partition(a);
   if (rc) return rc;
-  if (!a->query || !a->key_cache || !a->value_cache || !a->block_tables) return PA_ERR_NULL_POINTER;
-  if (a->block_size != 16 && a->block_size != 64 && a->block_size != 1024) return PA_ERR_UNSUPPORTED;
-  if (a->kv_dtype != PA_DTYPE_BF16 && a->kv_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
-  if (a->query_dtype != PA_DTYPE_BF16 && a->query_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
-  if (a->kv_quant_mode != PA_QUANT_NONE && (!a->key_scale || !a->value_scale)) return PA_ERR_NULL_POINTER;
-  if (a->query_quant_mode != PA_QUANT_NONE && !a->query_scale) return PA_ERR_NULL_POINTER;
-  if (a->kv_quant_mode < -1 || a->kv_quant_mode > 1 || a->query_quant_mode < -1 || a->query_quant_mode > 1)
-    return PA_ERR_UNSUPPORTED;
-  const int esz = a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
-  // 16-byte vector loads: every stride that moves a vector must keep it 16-byte aligned
-  if ((a->stride_k_b * esz) % 16 || (a->stride_k_h * esz) % 16 || (a->stride_k_c * esz) % 16 ||
-      (a->stride_v_b * esz) % 16 || (a->stride_v_h * esz) % 16 || (a->stride_v_2 * esz) % 16)
-    return PA_ERR_BAD_SHAPE;
-  const int qsz = a->query_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
-  if ((a->stride_q_s * qsz) % 16 || (a->stride_q_h * qsz) % 16) return PA_ERR_BAD_SHAPE;
-  if ((a->stride_tmp_g * 2) % 16 || (a->stride_tmp_p * 2) % 16 || (a->stride_tmp_h * 2) % 16 || (a->stride_tmp_s * 2) % 16 ||
-      (reinterpret_cast<uintptr_t>(a->tmp_output) & 15))
-    return PA_ERR_BAD_SHAPE;
-  if (a->kv_quant_mode == PA_QUANT_PER_TOKEN && (a->stride_kvscale_b % 4 || a->stride_kvscale_h % 4))
-    return PA_ERR_BAD_SHAPE;
-  if ((long long)(4 * 3 + 3) * a->stride_k_c * esz + 15 * 16 >= (1LL << 32)) return PA_ERR_BAD_SHAPE;
-  if ((reinterpret_cast<uintptr_t>(a->key_cache) | reinterpret_cast<uintptr_t>(a->value_cache) |
-       reinterpret_cast<uintptr_t>(a->query)) & 15)
-    return PA_ERR_BAD_SHAPE;
-
-  const int Ge = a->q_len * a->group_size;
-  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-  const bool pt = a->kv_quant_mode == PA_QUANT_PER_TOKEN;
-  if (a->kv_dtype == PA_DTYPE_FP8_E4M3FN) {
-    // constant in-page strides: block size 16 with the default dense layout
-    const bool bs16 = a->block_size == 16 && a->stride_k_c == 256 &&
-                      (a->v_transposed ? a->stride_v_2 == 2048 : a->stride_v_2 == 16);
-    if (use_shared_stream(a->kv_dtype, Ge)) {
-      if (bs16) return pt ? launch_partition_shared<true, true>(*a, stream) : launch_partition_shared<false, true>(*a, stream);
-      return pt ? launch_partition_shared<true, false>(*a, stream) : launch_partition_shared<false, false>(*a, stream);
-    }
-    if (bs16)
-      return pt ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, true>(*a, stream)
-                : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, true>(*a, stream);
-    return pt ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, false>(*a, stream)
-              : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, false>(*a, stream);
-  }
-  if (pt) return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
-  return launch_partition_tile<PA_DTYPE_BF16, false, false>(*a, stream);
+  return launch_partition(*a, choose_launch(*a), reinterpret_cast<hipStream_t>(hip_stream));
 }
 
 int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) { return launch_reduce(a, hip_stream, false); }
 
 int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
-  if (a && a->struct_size == sizeof(PaDecodeArgs) && !a->output) return PA_ERR_NULL_POINTER;
-  g_used_item_lists = false;
-  int rc = pa_decode_partition(a, hip_stream);
+  int rc = check_partition(a);
   if (rc) return rc;
-  // the partition kernel has written the rows of every sequence that fits in one partition itself
+  rc = check_reduce(a);  // before anything is launched
+  if (rc) return rc;
+  const LaunchChoice c = choose_launch(*a);
+  rc = launch_partition(*a, c, reinterpret_cast<hipStream_t>(hip_stream));
+  if (rc) return rc;
+  // the partition kernel has written the rows of every sequence that has a single partition itself
   if (a->max_num_partitions == 1 && !a->sinks) return PA_OK;
-  if (g_used_item_lists && !a->sinks && a->workspace_bytes >= full_workspace_bytes(a->num_seqs, a->max_num_partitions)) {
-    // (the stride checks of the reduce stage)
-    if (a->stride_out_h % 2 || a->stride_out_s % 2 || a->stride_tmp_g % 2 || a->stride_tmp_p % 2 || a->stride_tmp_h % 2 ||
-        a->stride_tmp_s % 2)
-      return PA_ERR_BAD_SHAPE;
-    return launch_reduce_listed(a, hip_stream);
-  }
+  if (c.listed_reduce) return launch_reduce_listed(a, hip_stream);
   return launch_reduce(a, hip_stream, true);
+}
+
+int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes) {
+  const int rc = check_partition(a);
+  if (rc) return rc;
+  if (!text || text_bytes <= 0) return PA_ERR_NULL_POINTER;
+  const LaunchChoice c = choose_launch(*a);
+  const char* cache = !c.fp8 ? "bf16" : (c.per_token ? "fp8 per-token" : "fp8");
+  if (c.shared)
+    snprintf(text, (size_t)text_bytes, "pa_partition_shared_kernel<%s, %s, %d ring slots, %d workgroups per CU> x %lld%s",
+             cache, c.bs16 ? "bs16" : "strided", c.per_token ? 3 : 2, c.per_cu, c.blocks, c.sorted ? ", sorted items" : "");
+  else
+    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves> x %lld%s", cache,
+             c.bs16 ? "bs16" : "strided", c.waves, c.blocks,
+             c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""));
+  return PA_OK;
 }
 
 int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
@@ -518,6 +550,20 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
     return PA_ERR_LAUNCH;
   }
   return pa_decode(&k, hip_stream);
+}
+
+int pa_debug_gather_probe(const PaDecodeArgs* a, int32_t* sink, void* hip_stream) {
+  const int rc = check_partition(a);
+  if (rc) return rc;
+  if (!sink) return PA_ERR_NULL_POINTER;
+  if (a->kv_dtype != PA_DTYPE_FP8_E4M3FN || a->block_size != 16 || a->stride_k_c != 256 || a->stride_v_2 != 16 ||
+      a->v_transposed)
+    return PA_ERR_UNSUPPORTED;
+  const long long blocks = (long long)a->num_seqs * a->num_kv_heads * a->max_num_partitions;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(pa_gather_probe_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(hip_stream), *a, sink);
+  return launch_status();
 }
 
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream) {

@@ -195,7 +195,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                         (int64_t)part * a.stride_tmp_p) * 2;
       char* op = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
-      const bool dir = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
+      const bool dir = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
       for (int r = row0 + kg; r < row0 + 16 * NT && r < Ge; r += 4) {
         if (li == 0) {
           a.max_logits[eo + r] = -INFINITY;
@@ -688,8 +688,10 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
   char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                      (int64_t)part * a.stride_tmp_p) * 2;
-  // a sequence that fits in one partition needs no merge: its partial is the result
-  const bool direct = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
+  // a sequence with one partition needs no merge: its partial is the result.  (With a partition axis of length
+  // 1 every sequence has one: a context longer than the partition is cut off at its end, as the partition axis
+  // cuts off longer contexts for any other length.)
+  const bool direct = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
   const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
   float l_tot[NT];

@@ -168,7 +168,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
   char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                      (int64_t)part * a.stride_tmp_p) * 2;
-  const bool direct = ctx <= a.partition_size && a.output != nullptr && a.sinks == nullptr;
+  const bool direct = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
   // ---- per-lane row bookkeeping ---------------------------------------------------------------------------------
   const bool has_alibi = a.alibi_slopes != nullptr;

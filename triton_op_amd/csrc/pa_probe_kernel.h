@@ -1,0 +1,89 @@
+// pa_gather_probe_kernel: a read-only probe of the partition kernel's memory access pattern.
+#ifndef PA_PROBE_KERNEL_H_
+#define PA_PROBE_KERNEL_H_
+
+#include "pa_common.h"
+
+namespace {
+
+// Reads what pa_partition_kernel<fp8, bs16, 4 waves> reads for the same arguments, in the same grouping and order
+// -- one workgroup of four waves per (sequence, partition, kv head), head fastest; wave w takes the 64-token
+// steps w, w + 4, ...; per step every lane issues eight 16-byte non-temporal loads of K (four 16-token tiles, two
+// loads each, lanes 0-15 = the tile's tokens, lane >> 4 = the chunk row) and eight of V (lanes 0-15 = 16 head dims,
+// lane >> 4 = the tile), one step ahead of the step whose bytes it folds together -- and does no arithmetic beyond
+// an XOR per loaded word.  What it reaches is what the memory system gives this gather pattern; the gap between it
+// and the partition kernel is what the kernel's arithmetic and its tail cost.
+// Block size 16, FP8 cache in the dense default layout only.  `sink` receives a word only if the fold of all the
+// bytes read is a value it cannot be (which keeps the loads alive without a store per workgroup).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void pa_gather_probe_kernel(const PaDecodeArgs a, int* sink) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, kg = lane >> 4;
+  const int Hkv = a.num_kv_heads;
+  const long long wid = blockIdx.x;
+  const int h = (int)(wid % Hkv);
+  const long long item = wid / Hkv;
+  const int b = (int)(item % a.num_seqs);
+  const int part = (int)(item / a.num_seqs);
+  const int ctx = sload_i32(a.context_lens + b);
+  const int wg_start = part * a.partition_size;
+  if (wg_start >= ctx) return;
+  const int wg_end = min(wg_start + a.partition_size, ctx);
+  const int wg_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
+  const int n_steps = wave < wg_steps ? (wg_steps - wave + 3) / 4 : 0;
+  if (n_steps == 0) return;
+  const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h;
+  const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h;
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const int last_tile_tok = (wg_end - 1) & ~15;
+  const uint32_t k_off = (uint32_t)(kg * 256 + li * 16);
+  struct Step {
+    u32x4 k[4][2];
+    u32x4 v[8];
+  };
+  auto issue = [&](Step& st, int tok0) {
+    int page[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int t = tok0 + 16 * j;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      page[j] = sload_i32(bt + (t >> 4));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const char* tb = kbase + (int64_t)page[j] * a.stride_k_b;
+      st.k[j][0] = load16_stream(tb + k_off);
+      st.k[j][1] = load16_stream(tb + k_off + 1024);
+    }
+    const int vp = kg == 0 ? page[0] : (kg == 1 ? page[1] : (kg == 2 ? page[2] : page[3]));
+    const char* tb = vbase + (int64_t)vp * a.stride_v_b;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) st.v[db] = load16_stream(tb + (li + 16 * db) * 16);
+  };
+  uint32_t fold = 0;
+  auto consume = [&](const Step& st) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int ld = 0; ld < 2; ++ld) fold ^= st.k[j][ld][0] ^ st.k[j][ld][1] ^ st.k[j][ld][2] ^ st.k[j][ld][3];
+#pragma unroll
+    for (int db = 0; db < 8; ++db) fold ^= st.v[db][0] ^ st.v[db][1] ^ st.v[db][2] ^ st.v[db][3];
+  };
+  int tok0 = wg_start + wave * kStepTokens;
+  Step cur, nxt;
+  issue(cur, tok0);
+  for (int s = 0; s + 1 < n_steps; ++s) {
+    tok0 += 4 * kStepTokens;
+    issue(nxt, tok0);
+    consume(cur);
+    cur = nxt;
+  }
+  consume(cur);
+  // FP8 cache bytes of real workloads never fold to this exact word in every lane at once
+  if (__builtin_amdgcn_ballot_w64(fold != 0x9e3779b9u) == 0) sink[lane] = (int)fold;
+}
+
+}  // namespace
+
+#endif  // PA_PROBE_KERNEL_H_

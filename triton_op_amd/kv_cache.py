@@ -39,6 +39,8 @@ def quantize_kv_cache_symmetric(
         raise ValueError("quantize_kv_cache_symmetric takes a bfloat16 cache")
     if not key_cache.is_cuda:
         raise ValueError("quantize_kv_cache_symmetric runs on the GPU only (kv_layout has the torch form)")
+    if value_cache.device != key_cache.device:
+        raise ValueError(f"value_cache is on {value_cache.device}, key_cache on {key_cache.device}")
     nblk, h, d, bs = value_cache.shape
     if tuple(key_cache.shape) != (nblk, h, d // 8, bs, 8) or d != 128:
         raise ValueError(f"key_cache shape {tuple(key_cache.shape)} does not match value_cache {tuple(value_cache.shape)}")
@@ -69,6 +71,12 @@ def kv_cache_write(
         raise ValueError("key and value must be bfloat16 [num_tokens, num_kv_heads, head_size]")
     if not key.is_cuda:
         raise ValueError("kv_cache_write runs on the GPU only")
+    # every pointer below is dereferenced by the kernel: a host tensor (a slot_mapping built on the CPU, say)
+    # would be a GPU memory fault, not an exception
+    for name, t_ in (("value", value), ("key_cache", key_cache), ("value_cache", value_cache),
+                     ("slot_mapping", slot_mapping), ("key_scale", key_scale), ("value_scale", value_scale)):
+        if t_ is not None and t_.device != key.device:
+            raise ValueError(f"{name} is on {t_.device}, key on {key.device}")
     t, h, d = key.shape
     if key.stride(2) != 1 or value.stride(2) != 1:
         raise ValueError("key/value must be contiguous in the last dimension")

@@ -80,6 +80,12 @@ class DecodePlan:
             stream = torch.cuda.current_stream(self.output.device).cuda_stream
         _cabi.check(self._lib.pa_decode(C.byref(self.args), C.c_void_p(stream)), "pa_decode")
 
+    def launch_info(self) -> str:
+        """The partition kernel instantiation, grid and item source the launch layer chooses for this call."""
+        buf = C.create_string_buffer(256)
+        _cabi.check(self._lib.pa_decode_launch_info(C.byref(self.args), buf, 256), "pa_decode_launch_info")
+        return buf.value.decode()
+
     def run_noalloc(self, stream: Optional[int] = None) -> None:
         """The same call through `pa_decode_noalloc`: the partition buffers and the workspace of this plan are
         left alone, the library uses its own per-GPU scratch array instead (64 MiB; larger calls raise).  Calls

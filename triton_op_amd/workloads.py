@@ -66,6 +66,7 @@ class Workload:
         kw = {}
         for k, v in self.__dict__.items():
             kw[k] = v.to(device) if isinstance(v, torch.Tensor) else v
+        kw["meta"] = {k: (v.to(device) if isinstance(v, torch.Tensor) else v) for k, v in self.meta.items()}
         return Workload(**kw)
 
 
