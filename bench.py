@@ -353,7 +353,7 @@ def _bench_decode(a) -> int:
 
     headline = a.workload or "c2"
     cfg = _Config(headline, dev, a.pools, a.partition_size, a.batch or None)
-    t = _time_config(lib, cfg, stream, a.steps, a.warmup, SETTLE_CALLS)
+    t = _time_config(lib, cfg, stream, a.steps, a.warmup, a.settle)
     wl0 = cfg.wl0
     achieved = cfg.kv_bytes / (t["kernel_us_avg"] * 1e-6) / 1e9
     traffic, traffic_note = _traffic(cfg)
@@ -369,7 +369,7 @@ def _bench_decode(a) -> int:
         "n_gpus": 1,
         "steps": a.steps,
         "warmup": a.warmup,
-        "settle_calls": SETTLE_CALLS,
+        "settle_calls": a.settle,
         "ms_per_step": round(t["wall_ms"], 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -450,7 +450,7 @@ def _bench_probe_gather(a) -> int:
         if rc:
             _cabi.check(rc, "pa_debug_gather_probe")
 
-    for i in range(SETTLE_CALLS):
+    for i in range(a.settle):
         call(i)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -463,7 +463,7 @@ def _bench_probe_gather(a) -> int:
     gbps = cfg.kv_bytes / (us * 1e-6) / 1e9
     print(json.dumps({
         "metric": "read-only gather probe of c2's page pattern (no arithmetic)", "value": round(gbps, 1), "unit": "GB/s",
-        "us_per_call": round(us, 2), "n_gpus": 1, "steps": a.steps, "warmup": SETTLE_CALLS, "ms_per_step": round(us / 1e3, 5),
+        "us_per_call": round(us, 2), "n_gpus": 1, "steps": a.steps, "warmup": a.settle, "ms_per_step": round(us / 1e3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "probe_gather_" + cfg.wl0.name, "bytes_per_call": cfg.kv_bytes,
                    "kv_pools_rotated": len(cfg.plans)},
@@ -589,6 +589,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="default run: the headline only")
     ap.add_argument("--batch", type=int, default=0, help="override the batch size (debugging only)")
+    ap.add_argument("--settle", type=int, default=SETTLE_CALLS,
+                    help="untimed calls before anything is measured (profiling runs lower it)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op shards by kv head or "

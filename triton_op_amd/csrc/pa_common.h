@@ -100,14 +100,22 @@ __device__ __forceinline__ float query_pow2_factor(float amax, float& inv) {
 }
 
 // max / sum over the four lanes {l, l^16, l^32, l^48}: v_permlane{16,32}_swap exchange 16- and
-// 32-lane halves inside the VALU (no LDS round trip)
+// 32-lane halves inside the VALU (no LDS round trip).  Written out as instructions: a swap of a register with
+// its own copy leaves {x[l], x[l^32]} (then {y[l], y[l^16]}) in the two registers of every lane, one move, one
+// swap and one max per level.  (From the builtins the compiler makes ten instructions of these six: it
+// re-canonicalises both results of every swap before it takes their maximum.)
 __device__ __forceinline__ float quad_row_max(float x) {
-  uint32_t u = __float_as_uint(x);
-  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  u = __float_as_uint(x);
-  auto b = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  float t;
+  asm("v_mov_b32 %1, %0\n\t"
+      "s_nop 1\n\t"
+      "v_permlane32_swap_b32 %0, %1\n\t"
+      "v_max_f32 %0, %0, %1\n\t"
+      "v_mov_b32 %1, %0\n\t"
+      "s_nop 1\n\t"
+      "v_permlane16_swap_b32 %0, %1\n\t"
+      "v_max_f32 %0, %0, %1"
+      : "+v"(x), "=&v"(t));
+  return x;
 }
 __device__ __forceinline__ float quad_row_sum(float x) {
   uint32_t u = __float_as_uint(x);

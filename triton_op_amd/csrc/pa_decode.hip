@@ -225,10 +225,11 @@ void launch_partition_tile(const PaDecodeArgs& k, const LaunchChoice& c, hipStre
 
 template <bool PT, bool BS16>
 void launch_partition_shared(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+  static const int pad = debug_switch("PA_DECODE_LDS_PAD", 0);  // experiment: unused LDS that lowers the occupancy
   if constexpr (PT)
-    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)c.blocks), dim3(256), 0, stream, k);
+    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)c.blocks), dim3(256), pad, stream, k);
   else
-    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)c.blocks), dim3(256), 0, stream, k);
+    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)c.blocks), dim3(256), pad, stream, k);
 }
 
 // stage 1 as chosen: the planning kernel when the items are to be sorted, then the partition kernel

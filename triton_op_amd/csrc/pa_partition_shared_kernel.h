@@ -237,8 +237,23 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   }
 
   const bool rs_nonneg = __builtin_amdgcn_ballot_w64(rscale < 0.f) == 0;
-  float v_run = 1e-30f;  // per-token V scales: running max of the scales seen so far
-  float m_run = -INFINITY;
+  // Online softmax against a reference that (almost) never moves.  l and the accumulator are kept relative to
+  // m_ref, the row's maximum at its first visible step, and in units of 2^k_ref (per-token V scales: the exponent
+  // of the largest V scale of that step).  Every later step produces its P relative to ITS OWN maximum and V-scale
+  // unit, rounded up to whole powers of two: P = exp2(x - m_ref - n) * v_scale * 2^(kPBits - k), n = ceil(max - m_ref)
+  // and k = exponent(largest V scale of the step), so P always fills the FP8 range, whatever the step's level.
+  // The power of two that brings the step's P V back to the reference, 2^(n + k - k_ref), is the E8M0 block scale of
+  // the P operand of the scaled MFMA -- exact, and free.  Nothing is rescaled per step: no exp2 of a maximum's
+  // movement, no multiplication of the 32 accumulator registers (with an exact running maximum some row of the
+  // sixteen moves on most steps of a long context).  The reference is re-based only when a step's level has run
+  // more than kMaxAhead powers of two ahead of it (f32 headroom), which ordinary data never does.
+  // (m_ref, l) stay a consistent pair; the epilogue restates l against the true maximum for the partition buffers.
+  constexpr int kPBits = 8;          // P is produced times 2^kPBits (at most 256; e4m3 reaches 448)
+  constexpr float kMaxAhead = 60.f;  // n and k - k_ref stay below this
+  float m_ref = -INFINITY;
+  float m_ref_safe = 0.f;   // m_ref, or 0 while it is -inf
+  float m_true = -INFINITY;
+  int k_ref = 0;            // per-token V scales: the accumulator's unit is 2^k_ref
   float l_run = 0.f;
   f32x4 acc[8];
 #pragma unroll
@@ -246,7 +261,8 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
 
   // ---- one step of 64 tokens out of LDS: the arithmetic of pa_partition_kernel's FP8 step, one row tile ----
   // HALF: this wave takes tiles 2*half, 2*half+1 of the step (32 tokens) instead of all four
-  auto compute = [&]<bool FULL, bool HALF>(const StepLds& st, int tok0) {
+  // QRES: the query has an FP8 residual (a bf16 query); an FP8 query is its own head
+  auto compute = [&]<bool FULL, bool HALF, bool QRES>(const StepLds& st, int tok0) {
     constexpr int T = HALF ? 2 : 4;       // 16-token tiles of the step this wave works on
     const int jb = HALF ? 2 * half : 0;   // the first of them
     f32x4 s[T];
@@ -257,13 +273,10 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
       const i32x8 ka = {(int)k0[0], (int)k0[1], (int)k0[2], (int)k0[3], (int)k1[0], (int)k1[1], (int)k1[2], (int)k1[3]};
       s[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
       s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qhi, s[jj], 0, 0, 0, 0, 0, 0);
-      if (q_has_residual) s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[jj], 0, 0, 0, 0, 0, 0);
+      if constexpr (QRES) s[jj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka, qlo, s[jj], 0, 0, 0, 0, 0, 0);
     }
-    // P is produced already multiplied by pmul = 256 / v_run (per-token V scales: v_run is the running
-    // maximum of the scales, P then also carries v_scale / v_run <= 1 and the accumulator is kept in units
-    // of v_run): log2(pmul) rides in the exponent's additive term, so it costs nothing per element
-    float vfac = 1.f, log2_pmul = 8.f, inv_pmul = 1.f / 256.f;
     f32x4 ks_cur[PER_TOKEN ? T : 1], vs_cur[PER_TOKEN ? T : 1];
+    int k = 0;  // per-token V scales: exponent of the step's largest V scale (the same in every lane)
     if constexpr (PER_TOKEN) {
       float vmx = 0.f;
 #pragma unroll
@@ -281,11 +294,8 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
         }
       }
       vmx = quad_row_max(vmx);
-      const float v_new = fmaxf(v_run, vmx);
-      vfac = v_new == v_run ? 1.f : v_run * __builtin_amdgcn_rcpf(v_new);
-      log2_pmul = 8.f - __builtin_amdgcn_logf(v_new);
-      inv_pmul = v_new * (1.f / 256.f);
-      v_run = v_new;
+      // vmx = f * 2^k, f in [0.5, 1); 0 for vmx == 0.  The same in every lane: kept in a scalar register
+      k = __builtin_amdgcn_readfirstlane(__builtin_amdgcn_frexp_expf(vmx));
     }
     // FULL: the row's scale (>= 0 on this path) is applied inside the exponent's fma, and to the maximum once
     float mx = -INFINITY;
@@ -306,11 +316,33 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     }
     mx = quad_row_max(mx);
     if constexpr (FULL) mx *= rscale;
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_safe);
-    m_run = m_new;
-    const float e_add = log2_pmul - m_safe;
+    m_true = fmaxf(m_true, mx);
+    // the rare step: a row sees its first key, or this step's level is too far ahead of the reference
+    float ahead = mx - m_ref;  // +inf at a row's first visible key, NaN while it has seen none (compares false)
+    if (__builtin_amdgcn_ballot_w64(ahead > kMaxAhead) != 0 || k - k_ref > (int)kMaxAhead) {
+      float alpha = 1.f;
+      if (ahead > kMaxAhead) {
+        alpha = fast_exp2(m_ref - mx);  // exp2(-inf) = 0 on the first visible step
+        m_ref = mx;
+        m_ref_safe = mx;
+        ahead = 0.f;
+      }
+      l_run *= alpha;
+      if constexpr (PER_TOKEN) {
+        // (the first step of all lands here with the accumulator still zero, and fixes the unit)
+        alpha *= __builtin_ldexpf(1.f, k_ref - k < -126 ? -126 : (k_ref - k > 126 ? 126 : k_ref - k));
+        k_ref = k;
+      }
+#pragma unroll
+      for (int db = 0; db < 8; ++db) acc[db] *= alpha;
+    }
+    // n: whole powers of two from the reference up (or down) to this step's maximum
+    const float nf = __builtin_ceilf(fmaxf(ahead, -kMaxAhead));  // (NaN, -inf: no visible key; every P is 0)
+    const int n = (int)nf;
+    const float e_add = (float)(kPBits - k) - m_ref_safe - nf;
+    // E8M0 block scale of P, 2^(p_scale - 127); n and k - k_ref are at most kMaxAhead each
+    int p_scale = n + (127 + k - k_ref);
+    p_scale = p_scale < 1 ? 1 : p_scale;
     const float e_mul = FULL ? rscale : 1.f;
     float psum = 0.f;
     uint32_t ph[4] = {0u, 0u, 0u, 0u}, pl[4] = {0u, 0u, 0u, 0u};  // (HALF: the tiles that are not this wave's hold P = 0)
@@ -339,43 +371,45 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
       ph[j] = (uint32_t)hi;
       pl[j] = (uint32_t)lo;
     }
-    l_run = l_run * alpha + psum * inv_pmul;
-    // the accumulator is rescaled only when some row's maximum (or the V scale unit) moved
-    const float alpha_acc = alpha * vfac;
-    if (__builtin_amdgcn_ballot_w64(alpha_acc != 1.f)) {
-#pragma unroll
-      for (int db = 0; db < 8; ++db) acc[db] *= alpha_acc;
-    }
+    // psum = sum of exp2(x - m_ref - n) * 2^(kPBits - k): back to the reference
+    l_run += __builtin_ldexpf(psum, n + k - kPBits);
 
-    // lane group kg holds, per tile j, tokens 4kg..4kg+3; the B operand of O^T += V^T P^T wants lane group
-    // kg to hold all 16 tokens of tile kg: a 4x4 transpose over (lane group, register)
-    quad_transpose(ph);
-    quad_transpose(pl);
-    // one 128-deep MFMA per 16 head dims covers head and residual of P at once: its reduction index runs
-    // over (tile kg's 16 tokens with P head, the same 16 tokens with P residual), so the A operand is the V
-    // bytes twice -- read from LDS twice, which costs no VALU slot
-    const i32x8 pb = {(int)ph[0], (int)ph[1], (int)ph[2], (int)ph[3], (int)pl[0], (int)pl[1], (int)pl[2], (int)pl[3]};
-    // after the transpose lane group kg holds P of the step's tile kg, or, HALF, of this wave's tile kg (kg < 2)
-    // and zeros (kg >= 2), which meet this wave's tiles' V bytes once more
-    const int vj = HALF ? jb + (kg & 1) : kg;
-    int nvalid = 16;
+    // One 128-deep MFMA per 16 head dims covers head and residual of P at once.  Its reduction index is laid out
+    // so that every lane's 32 bytes of V are 32 DIFFERENT tokens: lane groups 0 and 1 take the step's tiles 0-1
+    // and 2-3 against the head of P, lane groups 2 and 3 the same tiles against the residual.  Before, lane group
+    // g holds tokens 4g..4g+3 of every tile; two 4x4 (lane group x register) transposes bring every group the 16
+    // tokens of its first tile (pa) and of its second (pb).
+    // HALF: this wave's two tiles against head (group 0) and residual (group 2); groups 1 and 3 hold P = 0.
+    uint32_t pa[4], pb[4];
+    if constexpr (HALF) {
+      pa[0] = ph[0], pa[1] = 0u, pa[2] = pl[0], pa[3] = 0u;
+      pb[0] = ph[1], pb[1] = 0u, pb[2] = pl[1], pb[3] = 0u;
+    } else {
+      pa[0] = ph[0], pa[1] = ph[2], pa[2] = pl[0], pa[3] = pl[2];
+      pb[0] = ph[1], pb[1] = ph[3], pb[2] = pl[1], pb[3] = pl[3];
+    }
+    quad_transpose(pa);
+    quad_transpose(pb);
+    const i32x8 pv = {(int)pa[0], (int)pa[1], (int)pa[2], (int)pa[3], (int)pb[0], (int)pb[1], (int)pb[2], (int)pb[3]};
+    const int vj = HALF ? jb : 2 * (kg & 1);  // this lane group's first tile (the zero groups of HALF read real bytes too)
+    int nvalid0 = 16, nvalid1 = 16;
     if constexpr (!FULL) {
       // V bytes of tokens at or beyond ctx are zeroed (stale cache contents may decode to NaN)
-      nvalid = ctx - (tok0 + 16 * vj);
-      nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+      nvalid0 = ctx - (tok0 + 16 * vj);
+      nvalid0 = nvalid0 < 0 ? 0 : (nvalid0 > 16 ? 16 : nvalid0);
+      nvalid1 = ctx - (tok0 + 16 * vj + 16);
+      nvalid1 = nvalid1 < 0 ? 0 : (nvalid1 > 16 ? 16 : nvalid1);
     }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const u32x4* vp = &st.v[vj][16 * db + li];
-      typedef const volatile __attribute__((address_space(3))) u32x4* LdsVec;
-      u32x4 v0 = *vp;
-      u32x4 v1 = *(LdsVec)vp;  // a second LDS read, not a register copy
+      u32x4 v0 = st.v[vj][16 * db + li];
+      u32x4 v1 = st.v[vj + 1][16 * db + li];
       if constexpr (!FULL) {
-        v0 = keep_first_bytes(v0, nvalid);
-        v1 = keep_first_bytes(v1, nvalid);
+        v0 = keep_first_bytes(v0, nvalid0);
+        v1 = keep_first_bytes(v1, nvalid1);
       }
       const i32x8 va = {(int)v0[0], (int)v0[1], (int)v0[2], (int)v0[3], (int)v1[0], (int)v1[1], (int)v1[2], (int)v1[3]};
-      acc[db] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, pb, acc[db], 0, 0, 0, 0, 0, 0);
+      acc[db] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, pv, acc[db], 0, 0, 0, 127, 0, p_scale);
     }
   };
 
@@ -413,30 +447,31 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   // Three loops, each with one variant of the step (one loop with a choice inside would make the compiler
   // copy the whole accumulator state where the variants join, every step).  The waves of a workgroup may be
   // in different loops: all of them pass the same number of barriers.
+  // one pair of loops per variant: first the steps that need no masking, then the rest
+  auto run_steps = [&]<bool HALF, bool QRES>(int n_fast) {
+    while (s < n_fast) {
+      enter_step();
+      compute.template operator()<true, HALF, QRES>(stage[slot], tok0);
+      leave_step();
+    }
+    while (s < n_steps) {
+      enter_step();
+      compute.template operator()<false, HALF, QRES>(stage[slot], tok0);
+      leave_step();
+    }
+  };
   if (has_rows) {
     const int n_fast = rs_nonneg ? (n_full < n_steps ? n_full : n_steps) : 0;
     if (half_mode) {
-      while (s < n_fast) {
-        enter_step();
-        compute.template operator()<true, true>(stage[slot], tok0);
-        leave_step();
-      }
-      while (s < n_steps) {
-        enter_step();
-        compute.template operator()<false, true>(stage[slot], tok0);
-        leave_step();
-      }
+      if (q_has_residual)
+        run_steps.template operator()<true, true>(n_fast);
+      else
+        run_steps.template operator()<true, false>(n_fast);
     } else {
-      while (s < n_fast) {
-        enter_step();
-        compute.template operator()<true, false>(stage[slot], tok0);
-        leave_step();
-      }
-      while (s < n_steps) {
-        enter_step();
-        compute.template operator()<false, false>(stage[slot], tok0);
-        leave_step();
-      }
+      if (q_has_residual)
+        run_steps.template operator()<false, true>(n_fast);
+      else
+        run_steps.template operator()<false, false>(n_fast);
     }
   } else {
     while (s < n_steps) {
@@ -459,22 +494,24 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   };
 
   // ---- two waves per tile: the second hands its (m, l, O) to the first ------------------------------------------
-  float acc_unit = (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f);
+  float acc_unit = __builtin_ldexpf(1.f, k_ref - kPBits);
   if (half_mode) {
-    // per tile: m and l of the 16 rows (lanes 0..15) and the 32 accumulator registers of all 64 lanes, in units of 1
-    constexpr int kMergeFloats = 2 * 16 + 32 * 64;
+    // per tile: reference maximum, l and true maximum of the 16 rows (lanes 0..15) and the 32 accumulator
+    // registers of all 64 lanes, in units of 1
+    constexpr int kMergeFloats = 3 * 16 + 32 * 64;
     static_assert(sizeof(StepLds) * NB >= 2 * kMergeFloats * 4 + 2 * 16 * kORowBytes, "room for the merge buffers");
     float* mb = reinterpret_cast<float*>(&stage[0]) + (row0 >> 4) * kMergeFloats;
     if (has_rows && half == 1) {
       const float lt = quad_row_sum(l_run);
       if (kg == 0) {
-        mb[li] = m_run;
+        mb[li] = m_ref;
         mb[16 + li] = lt;
+        mb[32 + li] = m_true;
       }
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) mb[32 + (4 * db + r) * 64 + lane] = acc[db][r] * acc_unit;
+        for (int r = 0; r < 4; ++r) mb[48 + (4 * db + r) * 64 + lane] = acc[db][r] * acc_unit;
       }
     }
     __syncthreads();
@@ -486,15 +523,16 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     if (has_rows) {
       const float m1 = mb[li], l1 = mb[16 + li];
       const float l0 = quad_row_sum(l_run);
-      const float mm = fmaxf(m_run, m1);
+      const float mm = fmaxf(m_ref, m1);
       const float m_safe = mm == -INFINITY ? 0.f : mm;
-      const float w0 = fast_exp2(m_run - m_safe), w1 = fast_exp2(m1 - m_safe);  // exp2(-inf) = 0: a half that saw no key
+      const float w0 = fast_exp2(m_ref - m_safe), w1 = fast_exp2(m1 - m_safe);  // exp2(-inf) = 0: a half that saw no key
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[db][r] = acc[db][r] * (acc_unit * w0) + mb[32 + (4 * db + r) * 64 + lane] * w1;
+        for (int r = 0; r < 4; ++r) acc[db][r] = acc[db][r] * (acc_unit * w0) + mb[48 + (4 * db + r) * 64 + lane] * w1;
       }
-      m_run = mm;
+      m_ref = mm;
+      m_true = fmaxf(m_true, mb[32 + li]);
       // l_run becomes this lane's share of the merged sum: the row total in lane group 0, nothing elsewhere
       l_run = kg == 0 ? l0 * w0 + l1 * w1 : 0.f;
       acc_unit = 1.f;
@@ -509,16 +547,17 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   float l_tot = quad_row_sum(l_run);
   if (!row_ok) {
     l_tot = 0.f;
-    m_run = -INFINITY;
+    m_true = -INFINITY;
   }
   const float inv = l_tot > 0.f ? v_tensor_scale * acc_unit / l_tot : 0.f;
   if (row < Ge && kg == 0) {
-    a.max_logits[es_off + row] = m_run * (1.0f / kLog2e);
-    a.exp_sums[es_off + row] = l_tot;
+    // the partition buffers hold the true maximum and the sum taken against it
+    a.max_logits[es_off + row] = m_true * (1.0f / kLog2e);
+    a.exp_sums[es_off + row] = l_tot > 0.f ? l_tot * fast_exp2(m_ref - m_true) : 0.f;
   }
   // wave-private staging for the transposed store (two waves per tile: behind the merge buffers, one per tile)
   char* olds = reinterpret_cast<char*>(&stage[0]) +
-               (half_mode ? 2 * (2 * 16 + 32 * 64) * 4 + (row0 >> 4) * (16 * kORowBytes) : wave * (16 * kORowBytes));
+               (half_mode ? 2 * (3 * 16 + 32 * 64) * 4 + (row0 >> 4) * (16 * kORowBytes) : wave * (16 * kORowBytes));
   store_partial_tile(olds, acc, inv, tmp + (int64_t)row0 * a.stride_tmp_g * 2, a.stride_tmp_g * 2,
                      direct ? outp + (int64_t)row0 * a.stride_out_h * 2 : nullptr, a.stride_out_h * 2, Ge - row0, lane);
 }
