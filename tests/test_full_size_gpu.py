@@ -66,7 +66,19 @@ def test_full_size_configuration(cuda, name):
 
     # oracle on a few sequences
     order = torch.argsort(ctx)
-    ids = sorted({int(order[0]), int(order[len(order) // 2]), int(order[-1])})
+    ids = {int(order[0]), int(order[len(order) // 2]), int(order[-1])}
+    if wl.q_lens is not None:
+        # a ragged batch: the sample must hold a sequence of every query length (1 new token = one 16-row tile
+        # per kv head ... 4 new tokens = all four tiles of the shared-stream kernel's workgroup busy), each the
+        # sequence of that query length whose context is closest to the median (seconds on the CPU)
+        ql_cpu = wl.q_lens.cpu()
+        med = int(ctx[order[len(order) // 2]])
+        for qv in range(1, wl.q_len + 1):
+            cand = torch.nonzero(ql_cpu == qv).flatten()
+            assert cand.numel() > 0, f"no sequence with {qv} new tokens in {wl.name}"
+            ids.add(int(cand[torch.argmin((ctx[cand] - med).abs())]))
+        assert {int(ql_cpu[i]) for i in ids} >= set(range(1, wl.q_len + 1))
+    ids = sorted(ids)
     q, kc, vc, sctx, bt, ql, ks, vs = _subset_for_oracle(wl, ids)
     ref = O.paged_attention_decode_oracle(q, kc, vc, sctx, bt, wl.softmax_scale, ql, ks, vs, q_max=wl.q_len)
     torch.testing.assert_close(o[ids].cpu(), ref.float(), atol=2e-2, rtol=2e-2)

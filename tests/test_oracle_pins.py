@@ -241,3 +241,79 @@ def test_sink_term_closed_form():
     e0, e1, es = math.exp(2.0), math.exp(-1.0), math.exp(0.5)
     exp = torch.tensor([(e0 * 1.0 + e1 * 3.0) / (e0 + e1 + es), (e0 * 10.0 + e1 * -4.0) / (e0 + e1 + es)])
     torch.testing.assert_close(out.view(-1), exp, atol=1e-6, rtol=1e-6)
+
+
+def test_query_scale_equals_prescaled_query():
+    """An FP8 query with its scale must give what the f32 product (query * scale) gives as the query: per row
+    ([B, rows, 1]) and per tensor (0-dim).  A scale applied to the wrong row, or dropped, changes the logits."""
+    wl = _tiny("fp8", "token", q_len=2, hq=8, hkv=2, ctx=(7, 40))
+    q8, qs = L.pertoken_quant(wl.query.float())      # [B, rows, D] e4m3fn, [B, rows, 1]
+    assert qs.shape == (2, 2 * 2 * 4, 1) and float(qs.min()) != float(qs.max())
+    args = (wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale, 2, wl.key_scale,
+            wl.value_scale)
+    out_scaled = O.paged_attention_decode_oracle(q8, *args, query_scale=qs)
+    out_product = O.paged_attention_decode_oracle(q8.float() * qs, *args)
+    torch.testing.assert_close(out_scaled.float(), out_product.to(torch.bfloat16).float(), atol=0, rtol=0)
+    # the rows' scales differ, so swapping two rows' scales must change those rows
+    qs_swapped = qs.clone()
+    qs_swapped[:, [0, 5]] = qs[:, [5, 0]]
+    moved = O.paged_attention_decode_oracle(q8, *args, query_scale=qs_swapped)
+    assert not torch.equal(moved[:, 0], out_scaled[:, 0]) and torch.equal(moved[:, 1], out_scaled[:, 1])
+    # per tensor
+    s0 = torch.tensor(0.37)
+    out_t = O.paged_attention_decode_oracle(q8, *args, query_scale=s0)
+    out_p = O.paged_attention_decode_oracle(q8.float() * 0.37, *args)
+    torch.testing.assert_close(out_t.float(), out_p.to(torch.bfloat16).float(), atol=0, rtol=0)
+
+
+def test_sinks_follow_the_packed_row_order():
+    """sinks holds one logit per PACKED query row (kv head h, new token t, head g) -> h*q*G + t*G + g.  Checked
+    row by row against the closed form softmax with one extra, value-less column: a (h, t, g) permutation
+    applied in the wrong order pairs rows with other rows' sinks."""
+    q_len, hq, hkv = 3, 4, 2
+    g = hq // hkv
+    wl = _tiny("bf16", "none", q_len=q_len, hq=hq, hkv=hkv, ctx=(9, 21))
+    rows = hkv * q_len * g
+    sinks = torch.linspace(-2.0, 3.0, rows)  # all different
+    out = _oracle(wl, sinks=sinks)
+    kf, vf = O.flatten_key_cache(wl.key_cache), O.flatten_value_cache(wl.value_cache)
+    for b, ctx in enumerate((9, 21)):
+        k, v = O.gather_sequence(kf, vf, None, None, wl.block_tables[b], ctx, 16)  # [ctx, Hkv, D]
+        for h in range(hkv):
+            for t in range(q_len):
+                for gg in range(g):
+                    row = h * q_len * g + t * g + gg
+                    nvis = ctx - (q_len - 1 - t)
+                    s = (k[:nvis, h].double() @ wl.query[b, row].double()) * wl.softmax_scale
+                    m = max(float(s.max()), float(sinks[row]))
+                    e = torch.exp(s - m)
+                    o = (e[:, None] * v[:nvis, h].double()).sum(0) / (e.sum() + math.exp(float(sinks[row]) - m))
+                    torch.testing.assert_close(out[b, row].double(), o.to(torch.bfloat16).double(), atol=1e-2, rtol=1e-2)
+
+
+def test_alibi_in_the_two_stage_form_matches_the_end_to_end_oracle():
+    """partition_stage applies the ALiBi term per partition; merged by reduce_stage it must give the end-to-end
+    oracle's output (which test_alibi_matches_explicit_bias pins), for MTP rows and several partitions."""
+    wl = _tiny("fp8", "tensor", q_len=2, hq=4, hkv=2, bs=16, ctx=(300, 70, 513))
+    slopes = torch.tensor([0.3, 0.05, 0.011, 0.2])
+    end_to_end = _oracle(wl, alibi_slopes=slopes)
+    ml, es, to = O.partition_stage(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                   wl.softmax_scale, 2, wl.key_scale, wl.value_scale, slopes, 256)
+    merged = O.reduce_stage(ml, es, to, wl.context_lens, 256)
+    torch.testing.assert_close(merged.float(), end_to_end.float(), atol=2e-3, rtol=2 ** -7)
+    # and the term is really there: without it the result differs
+    plain = _oracle(wl)
+    assert float((plain.float() - end_to_end.float()).abs().max()) > 1e-2
+
+
+def test_error_stats_on_a_hand_computed_pair():
+    """error_stats restates compare_arrays (utils.py:50-56): max |a-b| and max |a-b| / (1 + |b|)."""
+    a = torch.tensor([[1.0, -2.0], [0.5, 10.0]])
+    b = torch.tensor([[1.5, -2.0], [0.0, 7.0]])
+    st = O.error_stats(a, b)
+    assert st["diff_abs_max"] == pytest.approx(3.0)
+    # |a-b| / (1+|b|) = 0.5/2.5, 0, 0.5/1, 3/8
+    assert st["max_diff_thr"] == pytest.approx(0.5)
+    assert st["nan_result"] == 0 and st["nan_ref"] == 0
+    st = O.error_stats(torch.tensor([float("nan"), 1.0]), torch.tensor([0.0, 1.0]))
+    assert st["nan_result"] == 1 and st["nan_ref"] == 0
