@@ -121,6 +121,7 @@ struct LaunchChoice {
   bool per_token;   // per-token kv scales
   bool bs16;        // constant in-page strides: block size 16 with the default dense layout
   int waves;        // waves per workgroup
+  int row_tiles;    // pa_partition_kernel: 16-row query tiles one workgroup computes in its pass over the pages (1 or 2)
   int per_cu;       // workgroups of this instantiation that fit a CU
   bool queue;       // a resident grid pulls live items from a counter in the workspace
   bool sorted;      // items come from the planning kernel's list in the workspace
@@ -137,6 +138,7 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
            (a.v_transposed ? a.stride_v_2 == 2048 : a.stride_v_2 == 16);
   c.shared = use_shared_stream(a.kv_dtype, ge);
   long long items;  // (sequence, partition) pairs times kv heads times row tiles
+  c.row_tiles = 1;
   if (c.shared) {
     // ring depth / waves per SIMD: without per-token scales the kernel fits 128 registers, and a fourth
     // workgroup per CU is worth more than a deeper ring (measured); with them it needs about 140
@@ -150,18 +152,22 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     // items of a ragged batch finish the launch alone, one slow wave each (256 sequences of 1..4096 tokens:
     // 196 us with one wave per workgroup against 179 us with four).
     static const int forced = debug_switch("PA_DECODE_WAVES", 0);
-    items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * ((ge + 15) / 16);
+    // A bf16 cache with more than 16 query rows per kv head: two row tiles per workgroup share one pass over the
+    // pages (one wave per SIMD then, with twice the accumulators); an FP8 cache has the shared-stream kernel.
+    static const int forced_tiles = debug_switch("PA_DECODE_ROW_TILES", 0);
+    c.row_tiles = forced_tiles > 0 ? forced_tiles : (!c.fp8 && ge > 16 ? 2 : 1);
+    items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * ((ge + 16 * c.row_tiles - 1) / (16 * c.row_tiles));
     int w = waves_for_partition_size(a.partition_size);
     if (forced > 0) {
       w = forced;
     } else {
-      const long long slots = 8LL * device_num_cus();
+      const long long slots = (c.row_tiles == 2 ? 4LL : 8LL) * device_num_cus();
       int need = 1;  // waves per workgroup that fill the slots, or keep a wave's share at 1024 tokens
       while (need < w && (items * need < slots || a.partition_size > 1024 * need)) need *= 2;
       w = need;
     }
     c.waves = w >= 4 ? 4 : (w >= 2 ? 2 : 1);
-    c.per_cu = 8 / c.waves;
+    c.per_cu = (c.row_tiles == 2 ? 4 : 8) / c.waves;
   }
   c.blocks = items;
   // The queued launch is used when the caller gave a workspace and per-sequence query lengths and a kv head has
@@ -172,7 +178,7 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
   // launched plainly.
   static const bool queue_off = debug_switch("PA_DECODE_QUEUE", 1) == 0;
   c.queue = !c.shared && !queue_off && a.workspace != nullptr && a.num_seqs <= kQueueMaxSeqs && a.q_lens != nullptr &&
-            ge > 16;
+            ge > 16 * c.row_tiles;
   if (c.queue) {
     const long long resident = (long long)device_num_cus() * c.per_cu;
     c.blocks = resident < items ? resident : items;
@@ -205,22 +211,22 @@ int launch_plan(const PaDecodeArgs& a, hipStream_t stream) {
 // pa_partition_kernel is instantiated with one 16-row query tile per workgroup (NT = 1): a bf16 cache with
 // more than 16 query rows per kv head gets one workgroup per tile (they read the same pages at the same time
 // from the same L2, and tiles that hold only padding rows cost nothing).
-template <int KVT, bool PT, bool BS16, int W>
+template <int NT, int KVT, bool PT, bool BS16, int W>
 void launch_partition_w(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
-  constexpr int OCC = 2;
+  constexpr int OCC = NT == 1 ? 2 : 1;
   if (c.queue)
-    hipLaunchKernelGGL((pa_partition_kernel<1, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
+    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
                        stream, k);
   else
-    hipLaunchKernelGGL((pa_partition_kernel<1, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
+    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
                        stream, k);
 }
 
-template <int KVT, bool PT, bool BS16>
+template <int NT, int KVT, bool PT, bool BS16>
 void launch_partition_tile(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
-  if (c.waves == 4) return launch_partition_w<KVT, PT, BS16, 4>(k, c, stream);
-  if (c.waves == 2) return launch_partition_w<KVT, PT, BS16, 2>(k, c, stream);
-  return launch_partition_w<KVT, PT, BS16, 1>(k, c, stream);
+  if (c.waves == 4) return launch_partition_w<NT, KVT, PT, BS16, 4>(k, c, stream);
+  if (c.waves == 2) return launch_partition_w<NT, KVT, PT, BS16, 2>(k, c, stream);
+  return launch_partition_w<NT, KVT, PT, BS16, 1>(k, c, stream);
 }
 
 template <bool PT, bool BS16>
@@ -245,18 +251,21 @@ int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t s
     k.flags = kFlagSortedItems;
   }
   if (!c.fp8) {
-    launch_partition_tile<PA_DTYPE_BF16, false, false>(k, c, stream);
+    if (c.row_tiles == 2)
+      launch_partition_tile<2, PA_DTYPE_BF16, false, false>(k, c, stream);
+    else
+      launch_partition_tile<1, PA_DTYPE_BF16, false, false>(k, c, stream);
   } else if (c.shared) {
     if (c.bs16)
       c.per_token ? launch_partition_shared<true, true>(k, c, stream) : launch_partition_shared<false, true>(k, c, stream);
     else
       c.per_token ? launch_partition_shared<true, false>(k, c, stream) : launch_partition_shared<false, false>(k, c, stream);
   } else if (c.bs16) {
-    c.per_token ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, true>(k, c, stream)
-                : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, true>(k, c, stream);
+    c.per_token ? launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, true, true>(k, c, stream)
+                : launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, false, true>(k, c, stream);
   } else {
-    c.per_token ? launch_partition_tile<PA_DTYPE_FP8_E4M3FN, true, false>(k, c, stream)
-                : launch_partition_tile<PA_DTYPE_FP8_E4M3FN, false, false>(k, c, stream);
+    c.per_token ? launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, true, false>(k, c, stream)
+                : launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, false, false>(k, c, stream);
   }
   return launch_status();
 }
@@ -480,8 +489,8 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
     snprintf(text, (size_t)text_bytes, "pa_partition_shared_kernel<%s, %s, %d ring slots, %d workgroups per CU> x %lld%s",
              cache, c.bs16 ? "bs16" : "strided", c.per_token ? 3 : 2, c.per_cu, c.blocks, c.sorted ? ", sorted items" : "");
   else
-    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves> x %lld%s", cache,
-             c.bs16 ? "bs16" : "strided", c.waves, c.blocks,
+    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s", cache,
+             c.bs16 ? "bs16" : "strided", c.waves, c.row_tiles == 2 ? ", 2 row tiles" : "", c.blocks,
              c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""));
   return PA_OK;
 }
