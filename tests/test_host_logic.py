@@ -293,3 +293,81 @@ def test_short_division_of_the_cache_writers_is_the_rounded_quotient(tmp_path):
     res = subprocess.run([str(exe), "8000"], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stdout + res.stderr
     assert " 0 mismatches; arbitrary" in res.stdout and res.stdout.rstrip().endswith("amax/448 0 mismatches")
+
+
+def _fake_args(*, b, hq, hkv, q, ctx, bs=16, ps, kv="fp8", per_token=False, ragged=False, workspace=True):
+    """A PaDecodeArgs with the shapes of a call and made-up, suitably aligned addresses: the launch layer's choice
+    is host arithmetic on the struct and dereferences nothing."""
+    a = _cabi.PaDecodeArgs()
+    a.struct_size = C.sizeof(_cabi.PaDecodeArgs)
+    g = hq // hkv
+    ge = q * g
+    esz = 1 if kv == "fp8" else 2
+    x = 16 // esz
+    base = 0x10000000
+    for i, name in enumerate(("output", "query", "key_cache", "value_cache", "context_lens", "block_tables", "exp_sums",
+                              "max_logits", "tmp_output")):
+        setattr(a, name, base + i * 0x1000000)
+    if ragged:
+        a.q_lens = base + 0x20000000
+    if kv == "fp8":
+        a.key_scale, a.value_scale = base + 0x30000000, base + 0x31000000
+    a.num_seqs, a.num_kv_heads, a.group_size, a.q_len, a.head_size, a.block_size = b, hkv, g, q, 128, bs
+    a.partition_size = ps
+    a.max_num_partitions = -(-ctx // ps)
+    a.query_dtype = _cabi.PA_DTYPE_BF16
+    a.kv_dtype = _cabi.PA_DTYPE_FP8_E4M3FN if kv == "fp8" else _cabi.PA_DTYPE_BF16
+    a.query_quant_mode = _cabi.PA_QUANT_NONE
+    a.kv_quant_mode = (_cabi.PA_QUANT_PER_TOKEN if per_token else _cabi.PA_QUANT_PER_TENSOR) if kv == "fp8" else _cabi.PA_QUANT_NONE
+    a.softmax_scale = 0.088
+    a.stride_out_h = a.stride_q_h = 128
+    a.stride_out_s = a.stride_q_s = 128 * hkv * ge
+    a.stride_k_c, a.stride_k_h = bs * x, 128 * bs
+    a.stride_k_b = a.stride_k_h * hkv
+    a.stride_v_2, a.stride_v_h, a.stride_v_b = bs, 128 * bs, 128 * bs * hkv
+    a.stride_bt_s = -(-ctx // bs)
+    P = a.max_num_partitions
+    a.stride_es_p, a.stride_es_h, a.stride_es_s = ge, ge * P, ge * P * hkv
+    a.stride_tmp_g, a.stride_tmp_p, a.stride_tmp_h, a.stride_tmp_s = 128, 128 * ge, 128 * ge * P, 128 * ge * P * hkv
+    a.stride_kvscale_h, a.stride_kvscale_b = bs, bs * hkv
+    if workspace:
+        a.workspace = base + 0x40000000
+        a.workspace_bytes = 64 + 8 * b * P + 4 * b
+    return a
+
+
+def test_launch_layer_choices(pa_lib):
+    """Which partition kernel, in which instantiation, over which grid: the launch layer's choice for the five
+    benchmark configurations at the tuning layer's partition size (256 compute units assumed when there is no
+    GPU) and for the cases that take another path."""
+    def info(**kw):
+        buf = C.create_string_buffer(256)
+        assert pa_lib.pa_decode_launch_info(C.byref(_fake_args(**kw)), buf, 256) == 0
+        return buf.value.decode()
+
+    # c2: one partition, four waves, 64 x 8 workgroups, no item list
+    assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=4096) == "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
+    # c2 at the reference's partition size: 16 x 512 one-wave workgroups, more than two rounds: sorted
+    assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=256) == "pa_partition_kernel<fp8, bs16, 1 waves> x 8192, sorted items"
+    # c4: 16 partitions per sequence, one round
+    assert info(b=4, hq=64, hkv=8, q=1, ctx=131072, ps=8192) == "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
+    # c3: block 1024 takes the run-time strides
+    assert info(b=128, hq=64, hkv=8, q=2, ctx=32768, bs=1024, ps=8192) == \
+        "pa_partition_kernel<fp8, strided, 4 waves> x 4096, sorted items"
+    # c5: 64 rows per kv head over an FP8 cache with per-token scales
+    assert info(b=256, hq=128, hkv=8, q=4, ctx=28856, ps=7424, per_token=True, ragged=True) == \
+        "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items"
+    assert info(b=128, hq=64, hkv=4, q=2, ctx=4096, ps=4096) == \
+        "pa_partition_shared_kernel<fp8, bs16, 2 ring slots, 4 workgroups per CU> x 512"
+    # c1: a bf16 cache, 8 rows, few workgroups
+    assert info(b=4, hq=8, hkv=1, q=1, ctx=1024, ps=1024, kv="bf16") == "pa_partition_kernel<bf16, strided, 4 waves> x 4"
+    # a bf16 cache with 32 rows per kv head: two row tiles per workgroup; ragged with a workspace: queued
+    assert info(b=128, hq=64, hkv=4, q=2, ctx=4096, ps=4096, kv="bf16") == \
+        "pa_partition_kernel<bf16, strided, 4 waves, 2 row tiles> x 512"
+    assert "queued items" in info(b=64, hq=128, hkv=8, q=4, ctx=4096, ps=4096, kv="bf16", ragged=True)
+    assert "queued items" not in info(b=64, hq=128, hkv=8, q=4, ctx=4096, ps=4096, kv="bf16", ragged=True, workspace=False)
+    # more sequences than the item tables of the queued / sorted launches hold: plain order, no error
+    assert info(b=5000, hq=8, hkv=1, q=1, ctx=4096, ps=256) == "pa_partition_kernel<fp8, bs16, 1 waves> x 80000"
+    # bad arguments are refused as by the launch itself
+    a = _fake_args(b=4, hq=8, hkv=1, q=1, ctx=1024, ps=300)
+    assert pa_lib.pa_decode_launch_info(C.byref(a), C.create_string_buffer(64), 64) == -4

@@ -579,3 +579,39 @@ def test_seeded_random_sweep(cuda, seed):
     assert not torch.isnan(out.float()).any()
     torch.testing.assert_close(out.float(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
     _check_stages(wl, res, res["partition_size"], slopes)
+
+
+@pytest.mark.parametrize("num_q_heads,q_len,scale_mode", [(16, 1, "tensor"), (32, 2, "token")])
+def test_understated_max_sequence_length_cuts_the_context_off(cuda, num_q_heads, q_len, scale_mode):
+    """max_sequence_length sizes the partition axis; a context that is longer than the axis covers is attended to up
+    to the end of the last partition only, whatever the length of the axis.  With an axis of length ONE that used to
+    leave the output rows unwritten (the partition kernel wrote them only for contexts inside the partition, and no
+    reduce kernel follows a single partition): now the single partition's result is the output, as the clamped
+    merge gives it for longer axes.  Checked against the oracle on the cut-off context (q_len 1: the cut is the
+    whole difference; q_len 2: the new tokens' causal offsets still count from the true context length, so only
+    the sequences that fit are compared with the oracle and the long one with the two-partition call's clamp)."""
+    import triton_op_amd as T
+
+    ctx_true = _ctx(700, 100, 512)
+    wl = _make(batch=3, num_q_heads=num_q_heads, num_kv_heads=2, context_lens=ctx_true, q_len=q_len, scale_mode=scale_mode)
+    g = wl.to(cuda)
+    for stated, ps in ((512, 512), (1024, 512)):
+        out = torch.full_like(g.query, float("nan"))
+        print(f"stated max_sequence_length={stated} partition_size={ps} heads={num_q_heads} q_len={q_len}", flush=True)
+        res = T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                                       g.softmax_scale, q_len, stated, torch.bfloat16, None, g.key_scale, g.value_scale,
+                                       partition_size=ps)
+        torch.cuda.synchronize()
+        assert res["maximum_logits"].shape[2] == stated // ps
+        assert not torch.isnan(out.float()).any()  # every row written
+        if stated == 1024:
+            ref = _oracle(wl)  # the axis covers every context: nothing is cut
+            torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)
+            continue
+        fits = [1, 2]
+        ref = _oracle(wl, seq_ids=fits)
+        torch.testing.assert_close(out[fits].float().cpu(), ref[fits].float(), atol=ATOL, rtol=RTOL)
+        if q_len == 1:
+            cut = type(wl)(**{**wl.__dict__, "context_lens": _ctx(512, 100, 512)})
+            ref_cut = _oracle(cut, seq_ids=[0])
+            torch.testing.assert_close(out[0].float().cpu(), ref_cut[0].float(), atol=ATOL, rtol=RTOL)
