@@ -6,6 +6,7 @@
     python bench.py --workload ref:B,Hq,Hkv,bs,qlen[,transv][,ctx=N]  one row of the reference harness's sweep
     python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1]
     python bench.py --workload probe_gather                          read-only probe of c2's page-gather pattern
+    python bench.py --workload probe_issue                           issue cost of the decode step's instructions
     python bench.py --workload kv_write | kv_quantize                the KV-cache write kernels, the step before the path
 
 A step is one call of the op (partition kernel + reduce kernel on one stream) on one batch of synthetic input
@@ -45,8 +46,8 @@ HBM_TRAFFIC = {
         "bytes": 541_400_000, "launch": "pa_partition_kernel<fp8, bs16, 4 waves> x 512",
         "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
     ("c5_ragged_mix", 7424): {
-        "bytes": 2_050_400_000,
-        "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 6512, sorted items",
+        "bytes": 2_050_500_000,
+        "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items",
         "profile": "profiles/pa_partition_shared_kernel_c5_hbm_traffic.md"},
 }
 
@@ -473,6 +474,54 @@ def _bench_probe_gather(a) -> int:
     return 0
 
 
+def _bench_probe_issue(a) -> int:
+    """What the instructions of the decode step cost a SIMD's issue port (pa_debug_issue_probe): nanoseconds per
+    instruction per wave with one and with three waves on every SIMD, and how far the matrix pipe runs beside the
+    vector ALU."""
+    import torch
+
+    from triton_op_amd import _cabi
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    lib = _cabi.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream(dev)
+    sh = C.c_void_p(stream.cuda_stream)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+    iters = 2000
+    names = {0: "v_fma_f32", 1: "v_mfma_f32_16x16x128_f8f6f4", 2: "16 MFMA + 128 v_fma_f32 interleaved (per iteration)",
+             3: "v_exp_f32", 4: "v_cvt_pk_fp8_f32", 5: "v_permlane32_swap"}
+    per_iter = {0: 128, 1: 16, 2: 1, 3: 128, 4: 128, 5: 128}
+    out = {}
+    for mode in range(6):
+        for waves in (1, 3):
+            def call():
+                _cabi.check(lib.pa_debug_issue_probe(mode, iters, cus * waves, C.c_void_p(sink.data_ptr()), sh), "probe")
+            call()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            call()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ns = e0.elapsed_time(e1) * 1e6 / (iters * per_iter[mode]) / waves
+            out[f"{names[mode]}, {waves} wave(s) per SIMD"] = round(ns, 2)
+    fma = out["v_fma_f32, 3 wave(s) per SIMD"]
+    print(json.dumps({
+        "metric": "issue cost of the decode step's instructions, ns per instruction per wave", "value": fma, "unit": "ns (v_fma_f32)",
+        "n_gpus": 1, "steps": iters, "warmup": 1, "ms_per_step": 0.0, "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 / fp8", "data": "synthetic", "config": {"workload": "probe_issue"},
+        "ns_per_instruction_per_wave": out,
+        "note": "a full-rate wave64 VALU instruction takes 4 shader cycles; the interleaved line is per iteration of "
+                "16 MFMAs + 128 fmas: max(MFMA alone, fma alone) if the matrix pipe ran entirely beside the vector ALU, "
+                "their sum if not at all"}, ensure_ascii=False))
+    return 0
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # the KV-cache write kernels
 # ---------------------------------------------------------------------------------------------------------------
@@ -600,6 +649,8 @@ def main() -> int:
         return _bench_kv_cache(a)
     if a.workload == "probe_gather":
         return _bench_probe_gather(a)
+    if a.workload == "probe_issue":
+        return _bench_probe_issue(a)
     return _bench_decode(a)
 
 

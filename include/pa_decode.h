@@ -277,6 +277,16 @@ int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_s
  */
 int pa_debug_gather_probe(const PaDecodeArgs* args, int32_t* sink, void* hip_stream);
 
+/*
+ * Measurement hook: the issue cost of the instructions the decode step is made of.  Launches `workgroups` workgroups
+ * of four waves (one per SIMD; 256 x n workgroups put n waves on every SIMD of a 256-CU GPU) that each run
+ * `iterations` x 128 instructions of one kind: mode 0 v_fma_f32 (the full-rate yardstick), 3 v_exp_f32,
+ * 4 v_cvt_pk_fp8_f32, 5 v_permlane32_swap; mode 1 runs iterations x 16 v_mfma_f32_16x16x128_f8f6f4, mode 2 the same
+ * 16 MFMAs with eight independent v_fma_f32 behind each (how far the matrix pipe runs beside the vector ALU).
+ * sink: at least 64 int32 of device memory (not written in practice).  Time it with events on the stream.
+ */
+int pa_debug_issue_probe(int32_t mode, int32_t iterations, int32_t workgroups, int32_t* sink, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "pa_decode_launch_info",
     "pa_debug_fp8_decode",
     "pa_debug_gather_probe",
+    "pa_debug_issue_probe",
     "pa_kv_cache_write",
     "pa_quantize_kv_cache",
 )
@@ -110,6 +111,8 @@ def load_library(path: str = None) -> C.CDLL:
         lib.pa_decode_launch_info.argtypes = [C.POINTER(PaDecodeArgs), C.c_char_p, C.c_int32]
         lib.pa_debug_gather_probe.restype = C.c_int
         lib.pa_debug_gather_probe.argtypes = [C.POINTER(PaDecodeArgs), C.c_void_p, C.c_void_p]
+        lib.pa_debug_issue_probe.restype = C.c_int
+        lib.pa_debug_issue_probe.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
         lib.pa_debug_fp8_decode.restype = C.c_int
         lib.pa_debug_fp8_decode.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
         lib.pa_kv_cache_write.restype = C.c_int

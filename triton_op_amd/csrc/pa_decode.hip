@@ -576,6 +576,23 @@ int pa_debug_gather_probe(const PaDecodeArgs* a, int32_t* sink, void* hip_stream
   return launch_status();
 }
 
+int pa_debug_issue_probe(int32_t mode, int32_t iterations, int32_t workgroups, int32_t* sink, void* hip_stream) {
+  if (!sink) return PA_ERR_NULL_POINTER;
+  if (iterations <= 0 || workgroups <= 0) return PA_ERR_BAD_SHAPE;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  const dim3 grid((unsigned)workgroups), block(256);
+  switch (mode) {
+    case 0: hipLaunchKernelGGL(pa_issue_probe_kernel<0>, grid, block, 0, stream, sink, iterations); break;
+    case 1: hipLaunchKernelGGL(pa_issue_probe_kernel<1>, grid, block, 0, stream, sink, iterations); break;
+    case 2: hipLaunchKernelGGL(pa_issue_probe_kernel<2>, grid, block, 0, stream, sink, iterations); break;
+    case 3: hipLaunchKernelGGL(pa_issue_probe_kernel<3>, grid, block, 0, stream, sink, iterations); break;
+    case 4: hipLaunchKernelGGL(pa_issue_probe_kernel<4>, grid, block, 0, stream, sink, iterations); break;
+    case 5: hipLaunchKernelGGL(pa_issue_probe_kernel<5>, grid, block, 0, stream, sink, iterations); break;
+    default: return PA_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream) {
   if (!codes || !out) return PA_ERR_NULL_POINTER;
   if (n <= 0) return PA_ERR_BAD_SHAPE;

@@ -84,6 +84,54 @@ void pa_gather_probe_kernel(const PaDecodeArgs a, int* sink) {
   if (__builtin_amdgcn_ballot_w64(fold != 0x9e3779b9u) == 0) sink[lane] = (int)fold;
 }
 
+// pa_issue_probe_kernel: what instructions of the decode step cost the issue port of a SIMD.  Every wave runs
+// `iters` iterations of 128 instructions of one kind on eight independent registers (MODE 0: v_fma_f32, the
+// full-rate yardstick; 3: v_exp_f32; 4: v_cvt_pk_fp8_f32; 5: v_permlane32_swap), or of 16 MFMAs
+// (v_mfma_f32_16x16x128_f8f6f4, MODE 1), or of the 16 MFMAs with eight independent v_fma_f32 behind each (MODE 2:
+// 128 fmas and 16 MFMAs per iteration; if the matrix pipe ran entirely beside the vector ALU this would take as long
+// as the longer of MODE 0 and MODE 1).  One workgroup of four waves is one wave per SIMD.
+template <int MODE>
+__global__ __launch_bounds__(256) void pa_issue_probe_kernel(int* sink, int iters) {
+  float x[8];
+  uint32_t u[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    x[i] = 0.001f * (float)(threadIdx.x + i + 1);
+    u[i] = threadIdx.x * 8u + (uint32_t)i;
+  }
+  i32x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (int)(threadIdx.x * 0x01010101u + (uint32_t)i);
+    b[i] = (int)(0x38383838u + (uint32_t)i);
+  }
+  f32x4 c[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if constexpr (MODE == 1 || MODE == 2)
+        c[r & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c[r & 3], 0, 0, 0, 0, 0, 0);
+      if constexpr (MODE != 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if constexpr (MODE == 0 || MODE == 2) x[i] = __builtin_fmaf(x[i], 1.0001f, 0.5f);
+          if constexpr (MODE == 3) x[i] = fast_exp2(x[i]);
+          if constexpr (MODE == 4) u[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(x[i], x[(i + 3) & 7], (int)u[i], false);
+          if constexpr (MODE == 5) {
+            auto t = __builtin_amdgcn_permlane32_swap(u[i], u[(i + 1) & 7], false, false);
+            u[i] = t[0];
+            u[(i + 1) & 7] = t[1];
+          }
+        }
+      }
+    }
+  }
+  float r = c[0][0] + c[1][1] + c[2][2] + c[3][3];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r += x[i] + (float)u[i];
+  if (r == 12345.678f) sink[threadIdx.x & 63] = (int)r;  // keeps the work alive
+}
+
 }  // namespace
 
 #endif  // PA_PROBE_KERNEL_H_
