@@ -78,8 +78,10 @@ int device_num_cus() {
 // Experiment switches.  They exist for tuning runs only and are dead unless the process was started with
 // PA_DECODE_DEBUG=1, so a serving process's launches never depend on stray environment variables:
 //   PA_DECODE_WAVES=n    waves per workgroup of pa_partition_kernel
+//   PA_DECODE_ROW_TILES=1  a bf16 cache with more than 16 query rows per kv head: one workgroup per 16-row tile
 //   PA_DECODE_QUEUE=0    no queued launch          PA_DECODE_SHARED=0   one workgroup per 16-row tile, always
 //   PA_DECODE_SORTED=0|1 never / always the sorted dispatch (when the workspace has room)
+//   PA_DECODE_LDS_PAD=n  unused LDS per workgroup of the shared-stream kernel (lowers its occupancy)
 // All are read once, at the first launch.
 int debug_switch(const char* name, int unset) {
   static const bool enabled = [] {
@@ -155,7 +157,7 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     // A bf16 cache with more than 16 query rows per kv head: two row tiles per workgroup share one pass over the
     // pages (one wave per SIMD then, with twice the accumulators); an FP8 cache has the shared-stream kernel.
     static const int forced_tiles = debug_switch("PA_DECODE_ROW_TILES", 0);
-    c.row_tiles = forced_tiles > 0 ? forced_tiles : (!c.fp8 && ge > 16 ? 2 : 1);
+    c.row_tiles = !c.fp8 && ge > 16 && forced_tiles != 1 ? 2 : 1;
     items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions * ((ge + 16 * c.row_tiles - 1) / (16 * c.row_tiles));
     int w = waves_for_partition_size(a.partition_size);
     if (forced > 0) {
