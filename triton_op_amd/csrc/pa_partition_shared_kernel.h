@@ -379,19 +379,21 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     // and 2-3 against the head of P, lane groups 2 and 3 the same tiles against the residual.  Before, lane group
     // g holds tokens 4g..4g+3 of every tile; two 4x4 (lane group x register) transposes bring every group the 16
     // tokens of its first tile (pa) and of its second (pb).
-    // HALF: this wave's two tiles against head (group 0) and residual (group 2); groups 1 and 3 hold P = 0.
+    // HALF: the wave has two tiles only, 64 of the 128 reduction slots: every lane group takes ONE tile in the first
+    // half of its 32 slots (groups 0/1: the two tiles against the head of P, groups 2/3 against the residual) and
+    // zeros in the second half, so one transpose and one LDS read of V per 16 head dims do.
     uint32_t pa[4], pb[4];
     if constexpr (HALF) {
-      pa[0] = ph[0], pa[1] = 0u, pa[2] = pl[0], pa[3] = 0u;
-      pb[0] = ph[1], pb[1] = 0u, pb[2] = pl[1], pb[3] = 0u;
+      pa[0] = ph[0], pa[1] = ph[1], pa[2] = pl[0], pa[3] = pl[1];
+      pb[0] = pb[1] = pb[2] = pb[3] = 0u;
     } else {
       pa[0] = ph[0], pa[1] = ph[2], pa[2] = pl[0], pa[3] = pl[2];
       pb[0] = ph[1], pb[1] = ph[3], pb[2] = pl[1], pb[3] = pl[3];
     }
     quad_transpose(pa);
-    quad_transpose(pb);
+    if constexpr (!HALF) quad_transpose(pb);
     const i32x8 pv = {(int)pa[0], (int)pa[1], (int)pa[2], (int)pa[3], (int)pb[0], (int)pb[1], (int)pb[2], (int)pb[3]};
-    const int vj = HALF ? jb : 2 * (kg & 1);  // this lane group's first tile (the zero groups of HALF read real bytes too)
+    const int vj = HALF ? jb + (kg & 1) : 2 * (kg & 1);  // this lane group's (first) tile
     int nvalid0 = 16, nvalid1 = 16;
     if constexpr (!FULL) {
       // V bytes of tokens at or beyond ctx are zeroed (stale cache contents may decode to NaN)
@@ -403,10 +405,11 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
       u32x4 v0 = st.v[vj][16 * db + li];
-      u32x4 v1 = st.v[vj + 1][16 * db + li];
+      u32x4 v1 = u32x4{0u, 0u, 0u, 0u};  // HALF: meets P = 0
+      if constexpr (!HALF) v1 = st.v[vj + 1][16 * db + li];
       if constexpr (!FULL) {
         v0 = keep_first_bytes(v0, nvalid0);
-        v1 = keep_first_bytes(v1, nvalid1);
+        if constexpr (!HALF) v1 = keep_first_bytes(v1, nvalid1);
       }
       const i32x8 va = {(int)v0[0], (int)v0[1], (int)v0[2], (int)v0[3], (int)v1[0], (int)v1[1], (int)v1[2], (int)v1[3]};
       acc[db] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, pv, acc[db], 0, 0, 0, 127, 0, p_scale);
