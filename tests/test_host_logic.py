@@ -347,8 +347,14 @@ def test_launch_layer_choices(pa_lib):
 
     # c2: one partition, four waves, 64 x 8 workgroups, no item list
     assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=4096) == "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
-    # c2 at the reference's partition size: 16 x 512 one-wave workgroups, more than two rounds: sorted
-    assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=256) == "pa_partition_kernel<fp8, bs16, 1 waves> x 8192, sorted items"
+    # c2 at the reference's partition size: 16 x 512 partitions for 2048 wave slots: one-wave workgroups of four each
+    assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 4 partitions per workgroup"
+    # ... of 1024 tokens: two each; and never more than the partition axis holds (3 partitions: one workgroup per sequence and head, four rounds of them: sorted)
+    assert info(b=128, hq=64, hkv=8, q=1, ctx=4096, ps=1024) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 2 partitions per workgroup"
+    assert info(b=1024, hq=64, hkv=8, q=1, ctx=768, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 8192, sorted items, 3 partitions per workgroup"
     # c4: 16 partitions per sequence, one round
     assert info(b=4, hq=64, hkv=8, q=1, ctx=131072, ps=8192) == "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
     # c3: block 1024 takes the run-time strides
@@ -367,7 +373,8 @@ def test_launch_layer_choices(pa_lib):
     assert "queued items" in info(b=64, hq=128, hkv=8, q=4, ctx=4096, ps=4096, kv="bf16", ragged=True)
     assert "queued items" not in info(b=64, hq=128, hkv=8, q=4, ctx=4096, ps=4096, kv="bf16", ragged=True, workspace=False)
     # more sequences than the item tables of the queued / sorted launches hold: plain order, no error
-    assert info(b=5000, hq=8, hkv=1, q=1, ctx=4096, ps=256) == "pa_partition_kernel<fp8, bs16, 1 waves> x 80000"
+    assert info(b=5000, hq=8, hkv=1, q=1, ctx=4096, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 20000, 4 partitions per workgroup"
     # bad arguments are refused as by the launch itself
     a = _fake_args(b=4, hq=8, hkv=1, q=1, ctx=1024, ps=300)
     assert pa_lib.pa_decode_launch_info(C.byref(a), C.create_string_buffer(64), 64) == -4

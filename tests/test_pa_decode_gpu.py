@@ -367,6 +367,66 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span",
+                         [("fp8", "tensor", 2, 1, False, 16, 256, 3), ("fp8", "token", 4, 2, False, 16, 256, 3),
+                          ("fp8", "tensor", 8, 2, False, 64, 256, 3), ("fp8", "tensor", 8, 2, False, 1024, 512, 2),
+                          ("bf16", "none", 16, 4, True, 16, 256, 4)])
+def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span):
+    """A caller-fixed small partition size and several rounds of one-wave workgroups: every workgroup then walks
+    several consecutive partitions in one pass over the pages (the launch layer says so) and writes one partial
+    result per partition.  The partition buffers are held against the oracle's partition stage, the merged result
+    against the oracle.  The partition axis (5 of 256 tokens, 3 of 512) is not a multiple of the span (3 or 4, 2),
+    contexts end on, before and
+    after partition boundaries, and in the ragged bf16 case a 32-row tile of some sequences holds padding rows
+    only (launched without a workspace, in plain order: with one, such batches take the queued launch)."""
+    import triton_op_amd as T
+
+    gen = torch.Generator().manual_seed(33)
+    batch = 200
+    ctx = torch.randint(1, 1101, (batch,), generator=gen, dtype=torch.int32)
+    ctx[:9] = torch.tensor([1, 255, 256, 257, 512, 768, 769, 1024, 1100], dtype=torch.int32)
+    ctx = torch.clamp(ctx, min=q_len)
+    q_lens = None
+    if ragged:
+        q_lens = torch.randint(1, q_len + 1, (batch,), generator=gen, dtype=torch.int32)
+        q_lens[:4] = torch.tensor([1, q_len, 2, 1], dtype=torch.int32)
+    wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, q_lens=q_lens,
+               kv_dtype=kv, scale_mode=scale_mode, block_size=block_size)
+    g = wl.to(cuda)
+    out = torch.full_like(g.query, float("nan"))
+    plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                         q_len, 1100, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
+                         query_lens=g.q_lens)
+    P = -(-1100 // ps)
+    assert plan.args.max_num_partitions == P
+    if ragged:
+        plan.args.workspace = None
+        plan.args.workspace_bytes = 0
+    # 8000 items for 2048 wave slots: three partitions each (4800 of 512 tokens: two); 16000 two-tile items for 1024
+    # slots: four, the most there is
+    assert f"{span} partitions per workgroup" in plan.launch_info(), plan.launch_info()
+    plan.exp_sums.fill_(float("nan"))
+    plan.max_logits.fill_(float("nan"))
+    plan.run()
+    torch.cuda.synchronize()
+    # partitions a sequence does not reach are not written; the oracle leaves them at its fill values
+    reach = (torch.arange(P)[None, :] * ps < ctx[:, None])  # [batch, P]
+    ml, es, to = O.partition_stage(
+        wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, None, ps, P, q_max=wl.q_len)
+    gml, ges, gto = plan.max_logits.cpu(), plan.exp_sums.cpu(), plan.tmp_output.float().cpu()
+    sel = reach[:, None, :, None].expand_as(ml)
+    fin = torch.isfinite(ml) & sel
+    assert torch.equal(gml[sel & ~torch.isfinite(ml)], ml[sel & ~torch.isfinite(ml)])
+    tight = kv == "bf16"
+    torch.testing.assert_close(gml[fin], ml[fin], atol=1e-4 if tight else 5e-4, rtol=1e-5 if tight else 5e-5)
+    torch.testing.assert_close(ges[sel], es[sel], atol=1e-4 if tight else 5e-4, rtol=1e-4 if tight else 1e-3)
+    sel_o = reach[:, None, :, None, None].expand_as(to)
+    torch.testing.assert_close(gto[sel_o], to[sel_o], atol=ATOL, rtol=RTOL)
+    assert not torch.isnan(out.float()).any()
+    torch.testing.assert_close(out.float().cpu(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+
+
 @pytest.mark.parametrize("group,q_len,scale_mode", [(8, 1, "tensor"), (16, 3, "token")])
 def test_item_list_reused_by_the_next_layer(cuda, group, q_len, scale_mode):
     """Two layers of one decode step share the sequence lengths and a workspace: the second is told to reuse the

@@ -22,6 +22,7 @@ typedef __attribute__((ext_vector_type(8))) int i32x8;
 constexpr int kHeadSize = 128;
 // PaDecodeArgs.flags as the kernels see it (the launch layer sets it in its own copy of the arguments)
 constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning kernel's item list
+constexpr int kFlagSpanShift = 20;         // bits 20..27: partitions a one-wave workgroup walks in one pass (0 = 1)
 // Workspace layout (int32 words): [0], [1] counters of the queued launch, [2] number of listed items,
 // [16 + 2i], [17 + 2i] sequence and partition index of item i.
 constexpr int kPlanHeaderWords = 16;
@@ -154,9 +155,8 @@ __device__ __forceinline__ u32x4 keep_first_bytes(u32x4 v, int n) {
 // rows of the partial output.  The tile is transposed through a wave-private LDS buffer so that every
 // store instruction writes four whole 256-byte rows (16 bytes per lane) instead of 32-byte fragments.
 constexpr int kORowBytes = 272;  // 256 B of bf16 + 16 B pad
-__device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, char* dst,
-                                                   int64_t row_stride_bytes, char* dst2, int64_t row_stride2_bytes,
-                                                   int rows_to_write, int lane) {
+// first half: the tile, scaled and rounded to bf16, into the LDS buffer (row li at li * kORowBytes)
+__device__ __forceinline__ void stage_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, int lane) {
   const int li = lane & 15, kg = lane >> 4;
 #pragma unroll
   for (int db = 0; db < 8; ++db) {
@@ -169,6 +169,11 @@ __device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+// second half: the staged rows to memory, four whole rows per store instruction (and to dst2, if given)
+__device__ __forceinline__ void copy_staged_tile(const char* lds, char* dst, int64_t row_stride_bytes, char* dst2,
+                                                 int64_t row_stride2_bytes, int rows_to_write, int lane) {
+  const int li = lane & 15, kg = lane >> 4;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = 4 * i + kg;
@@ -180,6 +185,12 @@ __device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
+}
+__device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, char* dst,
+                                                   int64_t row_stride_bytes, char* dst2, int64_t row_stride2_bytes,
+                                                   int rows_to_write, int lane) {
+  stage_partial_tile(lds, acc, inv, lane);
+  copy_staged_tile(lds, dst, row_stride_bytes, dst2, row_stride2_bytes, rows_to_write, lane);
 }
 
 // A sequence with no tokens at all (context length <= 0): nobody streams anything, and when the call has a

@@ -125,6 +125,7 @@ struct LaunchChoice {
   int waves;        // waves per workgroup
   int row_tiles;    // pa_partition_kernel: 16-row query tiles one workgroup computes in its pass over the pages (1 or 2)
   int per_cu;       // workgroups of this instantiation that fit a CU
+  int span;         // consecutive partitions a one-wave workgroup walks in one pass (1: one partition per workgroup)
   bool queue;       // a resident grid pulls live items from a counter in the workspace
   bool sorted;      // items come from the planning kernel's list in the workspace
   bool listed_reduce;  // ... and pa_decode's reduce stage walks the planning kernel's list of multi-partition sequences
@@ -185,6 +186,33 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     const long long resident = (long long)device_num_cus() * c.per_cu;
     c.blocks = resident < items ? resident : items;
   }
+  // One-wave workgroups in several rounds (a caller whose buffers fix a small partition size, the reference's 256):
+  // each workgroup walks `span` consecutive partitions in one pass over the pages and writes a partial result per
+  // partition, so the query set-up and the ramp of the page stream are paid once per span.  As many partitions
+  // as still leave a workgroup for every wave slot, no wave with more than 2048 tokens, and at most four (the
+  // partial results wait in LDS for the end of the pass).
+  c.span = 1;
+  static const int forced_span = debug_switch("PA_DECODE_SPAN", 0);  // 1 switches it off
+  if (!c.shared && !c.queue && c.waves == 1 && a.max_num_partitions > 1) {
+    const long long slots = (c.row_tiles == 2 ? 4LL : 8LL) * device_num_cus();
+    long long span = items / slots;
+    const long long cap = 2048 / a.partition_size;
+    span = span > cap ? cap : span;
+    // (measured, kernel + reduce, against one partition per workgroup: 64 sequences x 8 kv heads x 4096 tokens at
+    // 256: 110 -> 95 us; 4 x 8 x 131072 at 256: 235 -> 223 us; 256 x 8 x 2048 at 512: 200 -> 180 us; 512 x 8 x 4096
+    // at 256, eight rounds: 829 -> 808 us; pages of 1024 tokens, 128 x 8 x 16384, at 512: 847 -> 832 us, but at
+    // 256: 920 -> 936 us, so not there)
+    if (a.block_size > 64 && a.partition_size < 512) span = 1;
+    if (forced_span > 0) span = forced_span;
+    span = span > a.max_num_partitions ? a.max_num_partitions : span;
+    span = span > 4 ? 4 : span;
+    if (span >= 2) {
+      c.span = (int)span;
+      const long long coarse = (a.max_num_partitions + span - 1) / span;
+      items = items / a.max_num_partitions * coarse;
+      c.blocks = items;
+    }
+  }
   // The sorted dispatch pays a small extra kernel, and ordering only matters when workgroups are handed out in
   // several rounds: it is used when the launch has more than twice as many workgroups as the GPU holds at once
   // and the caller's workspace has room for the list (batches of more than kPlanMaxSeqs sequences, the planning
@@ -193,7 +221,9 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
   c.sorted = !c.queue && sorted_mode != 0 && a.workspace != nullptr && a.num_seqs <= kPlanMaxSeqs &&
              a.workspace_bytes >= plan_workspace_bytes(a.num_seqs, a.max_num_partitions) &&
              (sorted_mode == 1 || items > 2LL * device_num_cus() * c.per_cu);
-  c.listed_reduce = c.sorted && !a.sinks &&
+  // (with several partitions per workgroup the planning kernel lists those coarser items, and its list of the
+  // sequences with more than one of them is not the list of the sequences the reduce stage has to merge)
+  c.listed_reduce = c.sorted && c.span == 1 && !a.sinks &&
                     a.workspace_bytes >= full_workspace_bytes(a.num_seqs, a.max_num_partitions);
   return c;
 }
@@ -247,11 +277,15 @@ int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t s
   k.flags = 0;
   if (c.sorted) {
     if (!(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST)) {
-      const int rc = launch_plan(a, stream);
+      PaDecodeArgs items = a;  // what the planning kernel lists: a workgroup's `span` partitions are one item
+      items.partition_size = a.partition_size * c.span;
+      items.max_num_partitions = (a.max_num_partitions + c.span - 1) / c.span;
+      const int rc = launch_plan(items, stream);
       if (rc) return rc;
     }
     k.flags = kFlagSortedItems;
   }
+  if (c.span > 1) k.flags |= c.span << kFlagSpanShift;
   if (!c.fp8) {
     if (c.row_tiles == 2)
       launch_partition_tile<2, PA_DTYPE_BF16, false, false>(k, c, stream);
@@ -491,9 +525,13 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
     snprintf(text, (size_t)text_bytes, "pa_partition_shared_kernel<%s, %s, %d ring slots, %d workgroups per CU> x %lld%s",
              cache, c.bs16 ? "bs16" : "strided", c.per_token ? 3 : 2, c.per_cu, c.blocks, c.sorted ? ", sorted items" : "");
   else
-    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s", cache,
+  {
+    char span_text[48] = "";
+    if (c.span > 1) snprintf(span_text, sizeof(span_text), ", %d partitions per workgroup", c.span);
+    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s%s", cache,
              c.bs16 ? "bs16" : "strided", c.waves, c.row_tiles == 2 ? ", 2 row tiles" : "", c.blocks,
-             c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""));
+             c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""), span_text);
+  }
   return PA_OK;
 }
 

@@ -65,6 +65,13 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 
   __shared__ __attribute__((aligned(16))) char p_lds[FP8MATH ? 1 : WAVES][FP8MATH ? 1 : NT][FP8MATH ? 16 : 16 * kPRowBytes];
   __shared__ __attribute__((aligned(16))) char o_lds[1][16 * kORowBytes];
+  // SPAN: the partial results of the partitions a workgroup has left behind wait here for the end of the pass
+  // (stores in the middle of the page stream would hold up the loads issued after them: memory operations of a
+  // wave retire in order).  Per partition and row tile: 16 staged bf16 rows, then 16 maxima and 16 sums.
+  constexpr int kSpanMax = 4;
+  constexpr int kSpanSlotBytes = 16 * kORowBytes + 2 * 16 * 4;
+  constexpr bool kSpanCapable = WAVES == 1 && !QUEUE;
+  __shared__ __attribute__((aligned(16))) char span_lds[kSpanCapable ? (kSpanMax - 1) * NT * kSpanSlotBytes : 16];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -121,6 +128,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     total_items = q_cum[a.num_seqs] * Hkv;
   }
 
+  // SPAN (one-wave workgroups, plain or sorted launch order): the workgroup walks `span` consecutive partitions in one pass
+  // over the pages, and writes the partial result of each as it crosses into the next.  For callers whose buffers
+  // fix a small partition size (the reference's constant 256): the query set-up and the ramp of the page stream
+  // are paid once per span instead of once per four steps.
+  int span = 1;
+  if constexpr (kSpanCapable) {
+    span = (a.flags >> kFlagSpanShift) & 0xff;
+    span = span < 1 ? 1 : (span > kSpanMax ? kSpanMax : span);
+  }
+
   for (;;) {  // one pass without the queue
   int h, rt, b, part, tiles_b = RT;
   if constexpr (QUEUE) {
@@ -155,10 +172,10 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
       if (item >= sload_i32(a.workspace + 2)) return;
       b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);
-      part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1);
+      part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1) * span;
     } else {
       b = (int)(item % a.num_seqs);
-      part = (int)(item / a.num_seqs);
+      part = (int)(item / a.num_seqs) * span;
     }
   }
   const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
@@ -176,7 +193,8 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     }
     break;
   }
-  const int wg_end = min(wg_start + a.partition_size, ctx);
+  const int span_here = min(span, P - part);  // partitions of this workgroup that the buffers have room for
+  const int wg_end = min(wg_start + span_here * a.partition_size, ctx);
   // The waves take the partition's 64-token steps round robin (wave w: steps w, w + WAVES, ...), so at any
   // time the workgroup reads WAVES * 64 consecutive tokens: with large blocks that is whole 128-byte lines of
   // every V row and long runs of every K chunk row, requested by the waves together.  A wave with no step
@@ -191,18 +209,25 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   if (row0 >= rows_valid) {
     // only padding rows (a ragged batch): nothing to stream; the rows read as "no visible key"
     if (wave == 0) {
-      const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
-      char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
-                                        (int64_t)part * a.stride_tmp_p) * 2;
-      char* op = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
-      const bool dir = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
-      for (int r = row0 + kg; r < row0 + 16 * NT && r < Ge; r += 4) {
-        if (li == 0) {
-          a.max_logits[eo + r] = -INFINITY;
-          a.exp_sums[eo + r] = 0.f;
+      auto write_padding = [&](int pp) {
+        const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)pp * a.stride_es_p;
+        char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                          (int64_t)pp * a.stride_tmp_p) * 2;
+        char* op = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+        const bool dir = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
+        for (int r = row0 + kg; r < row0 + 16 * NT && r < Ge; r += 4) {
+          if (li == 0) {
+            a.max_logits[eo + r] = -INFINITY;
+            a.exp_sums[eo + r] = 0.f;
+          }
+          *reinterpret_cast<u32x4*>(tp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
+          if (dir) *reinterpret_cast<u32x4*>(op + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
         }
-        *reinterpret_cast<u32x4*>(tp + (int64_t)r * a.stride_tmp_g * 2 + li * 16) = u32x4{0, 0, 0, 0};
-        if (dir) *reinterpret_cast<u32x4*>(op + (int64_t)r * a.stride_out_h * 2 + li * 16) = u32x4{0, 0, 0, 0};
+      };
+      if constexpr (WAVES == 1 && !QUEUE) {
+        for (int pp = part; pp * a.partition_size < wg_end; ++pp) write_padding(pp);  // every partition of the span
+      } else {
+        write_padding(part);
       }
     }
     break;
@@ -325,22 +350,39 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   bf16x8 qreg[NT][4];
   {
     const char* q_ptr = (const char*)a.query;
+    // all loads of the tile rows go out together (one choice of the query's type around them, not one inside each:
+    // the compiler would wait for every load before it issues the next)
+    const bool q_bf16 = a.query_dtype == PA_DTYPE_BF16;
+    u32x4 raw[NT][4];
+    bool ok[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       const int row = row0 + 16 * nt + li;
-      const bool ok = row < rows_valid;
-      const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (ok ? row : 0)) * a.stride_q_h;
+      ok[nt] = row < rows_valid;
+      const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (ok[nt] ? row : 0)) * a.stride_q_h;
+      if (q_bf16) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
+          raw[nt][s] = load16(q_ptr + (e0 + dim) * 2);
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
+          const u32x2 r8 = *reinterpret_cast<const u32x2*>(q_ptr + e0 + dim);
+          raw[nt][s] = u32x4{r8[0], r8[1], 0, 0};
+        }
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const int dim = kFp8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
         Bf16x8Bits q;
-        if (a.query_dtype == PA_DTYPE_BF16) {
-          q.u = load16(q_ptr + (e0 + dim) * 2);
-        } else {
-          u32x2 raw = *reinterpret_cast<const u32x2*>(q_ptr + e0 + dim);
-          q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
-        }
-        if (!ok) q.u = u32x4{0, 0, 0, 0};
+        q.u = raw[nt][s];
+        if (!q_bf16) q.v = fp8x8_to_bf16x8(raw[nt][s][0], raw[nt][s][1]);
+        if (!ok[nt]) q.u = u32x4{0, 0, 0, 0};
         qreg[nt][s] = q.v;
       }
     }
@@ -400,18 +442,21 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       }
     }
   }
-  float v_run = 1e-30f;  // FP8 math with per-token V scales: running max of the scales seen so far
-
+  float v_run;          // FP8 math with per-token V scales: running max of the scales seen so far
   float m_run[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
   float l_run[NT];      // this lane's share of the running sum of exp2(s - m)
   f32x4 acc[NT][8];     // O^T: acc[nt][db][r] is head dim 16*db + 4*kg + r of query row 16*nt + li
+  auto reset_state = [&]() {
+    v_run = 1e-30f;
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    m_run[nt] = -INFINITY;
-    l_run[nt] = 0.f;
+    for (int nt = 0; nt < NT; ++nt) {
+      m_run[nt] = -INFINITY;
+      l_run[nt] = 0.f;
 #pragma unroll
-    for (int db = 0; db < 8; ++db) acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+      for (int db = 0; db < 8; ++db) acc[nt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  reset_state();
 
   char* plds = &p_lds[wave][0][0];
 
@@ -646,6 +691,38 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     n_full = (min_limit - part_start - kStepTokens) / kWaveStride + 1;
   int sidx = 0;
   int tok0 = part_start;
+  // SPAN: the partition being accumulated, and the steps left in it; at the boundary its partial result is
+  // set aside in LDS and the running state starts again (the page stream does not notice)
+  int part_cur = part;
+  const int steps_per_part = a.partition_size / kStepTokens;
+  int steps_left_in_part = steps_per_part;
+  auto cross_boundary = [&]() {
+    if constexpr (kSpanCapable) {
+      if (span > 1 && --steps_left_in_part == 0) {
+        // (the one-wave epilogue below, up to the staging in LDS, for a partition that is not the workgroup's last)
+        const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          char* slot = &span_lds[0] + ((part_cur - part) * NT + nt) * kSpanSlotBytes;
+          float l_tot = quad_row_sum(l_run[nt]);
+          float m_out = m_run[nt];
+          if (row0 + 16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
+            l_tot = 0.f;
+            m_out = -INFINITY;
+          }
+          const float inv = l_tot > 0.f ? v_tensor_scale * acc_unit / l_tot : 0.f;
+          if (kg == 0) {
+            reinterpret_cast<float*>(slot + 16 * kORowBytes)[li] = m_out * (1.0f / kLog2e);
+            reinterpret_cast<float*>(slot + 16 * kORowBytes)[16 + li] = l_tot;
+          }
+          stage_partial_tile(slot, acc[nt], inv, lane);
+        }
+        reset_state();
+        ++part_cur;
+        steps_left_in_part = steps_per_part;
+      }
+    }
+  };
   if (active) {
     const int n_fast = n_full < n_steps - 1 ? n_full : n_steps - 1;
     Pages pg_next = load_pages(part_start + kWaveStride);
@@ -668,26 +745,27 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       step.template operator()<true, true>(buf_a, tok0, pg_next);
       pg_next = pg_after;
       tok0 += kWaveStride;
+      cross_boundary();
     }
     for (; sidx < n_steps - 1; ++sidx) {
       const Pages pg_after = load_pages(tok0 + 2 * kWaveStride);
       step.template operator()<false, true>(buf_a, tok0, pg_next);
       pg_next = pg_after;
       tok0 += kWaveStride;
+      cross_boundary();
     }
     if (n_full >= n_steps)
       step.template operator()<true, false>(buf_a, tok0, pg_next);
     else
       step.template operator()<false, false>(buf_a, tok0, pg_next);
   }
-
   // ---- epilogue ------------------------------------------------------------------------------------------------
   // max_logits holds the maximum of the scaled logits in the natural-log domain, exp_sums the
   // un-normalised sum, tmp_output the normalised bf16 partial.  For a sequence that fits in one partition the
   // partial is the result, and it is written to output as well.
-  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part_cur * a.stride_es_p;
   char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
-                                     (int64_t)part * a.stride_tmp_p) * 2;
+                                     (int64_t)part_cur * a.stride_tmp_p) * 2;
   // a sequence with one partition needs no merge: its partial is the result.  (With a partition axis of length
   // 1 every sequence has one: a context longer than the partition is cut off at its end, as the partition axis
   // cuts off longer contexts for any other length.)
@@ -776,6 +854,26 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         }
       }
       if (nt + 1 < NT) __syncthreads();
+    }
+  }
+  if constexpr (kSpanCapable) {
+    // SPAN: the partitions left behind on the way (a sequence that crosses a boundary has more than one
+    // partition: nothing of it goes to `output` directly)
+    for (int pc = part; pc < part_cur; ++pc) {
+      const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)pc * a.stride_es_p;
+      char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                                        (int64_t)pc * a.stride_tmp_p) * 2;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const char* slot = &span_lds[0] + ((pc - part) * NT + nt) * kSpanSlotBytes;
+        const int row = row0 + 16 * nt + li;
+        if (row < Ge && kg == 0) {
+          a.max_logits[eo + row] = reinterpret_cast<const float*>(slot + 16 * kORowBytes)[li];
+          a.exp_sums[eo + row] = reinterpret_cast<const float*>(slot + 16 * kORowBytes)[16 + li];
+        }
+        copy_staged_tile(slot, tp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2, a.stride_tmp_g * 2, nullptr, 0,
+                         Ge - row0 - 16 * nt, lane);
+      }
     }
   }
   if constexpr (QUEUE) {

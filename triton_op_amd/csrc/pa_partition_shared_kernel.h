@@ -196,17 +196,26 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   {
     const char* q_ptr = (const char*)a.query;
     const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (row_ok ? row : 0)) * a.stride_q_h;
+    // the four loads of a row's 32 elements go out together (one choice of the query's type around them, not one
+    // inside each: the compiler would wait for every load before it issues the next)
+    u32x4 raw[4];
+    const bool q_bf16 = a.query_dtype == PA_DTYPE_BF16;
+    if (q_bf16) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) raw[s] = load16(q_ptr + (e0 + 64 * (s >> 1) + 16 * kg + 8 * (s & 1)) * 2);
+    } else {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x2 r8 = *reinterpret_cast<const u32x2*>(q_ptr + e0 + 64 * (s >> 1) + 16 * kg + 8 * (s & 1));
+        raw[s] = u32x4{r8[0], r8[1], 0, 0};
+      }
+    }
     float f[32];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int dim = 64 * (s >> 1) + 16 * kg + 8 * (s & 1);
       Bf16x8Bits q;
-      if (a.query_dtype == PA_DTYPE_BF16) {
-        q.u = load16(q_ptr + (e0 + dim) * 2);
-      } else {
-        u32x2 raw = *reinterpret_cast<const u32x2*>(q_ptr + e0 + dim);
-        q.v = fp8x8_to_bf16x8(raw[0], raw[1]);
-      }
+      q.u = raw[s];
+      if (!q_bf16) q.v = fp8x8_to_bf16x8(raw[s][0], raw[s][1]);
       if (!row_ok) q.u = u32x4{0, 0, 0, 0};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
