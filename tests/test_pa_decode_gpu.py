@@ -367,18 +367,19 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
-@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span",
-                         [("fp8", "tensor", 2, 1, False, 16, 256, 3), ("fp8", "token", 4, 2, False, 16, 256, 3),
-                          ("fp8", "tensor", 8, 2, False, 64, 256, 3), ("fp8", "tensor", 8, 2, False, 1024, 512, 2),
-                          ("bf16", "none", 16, 4, True, 16, 256, 4)])
-def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span):
+@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span,alibi",
+                         [("fp8", "tensor", 2, 1, False, 16, 256, 3, False), ("fp8", "token", 4, 2, False, 16, 256, 3, False),
+                          ("fp8", "tensor", 8, 2, False, 64, 256, 3, False), ("fp8", "tensor", 8, 2, False, 1024, 512, 2, False),
+                          ("bf16", "none", 16, 4, True, 16, 256, 4, False), ("fp8", "token", 8, 1, False, 16, 256, 3, True)])
+def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span, alibi):
     """A caller-fixed small partition size and several rounds of one-wave workgroups: every workgroup then walks
     several consecutive partitions in one pass over the pages (the launch layer says so) and writes one partial
     result per partition.  The partition buffers are held against the oracle's partition stage, the merged result
     against the oracle.  The partition axis (5 of 256 tokens, 3 of 512) is not a multiple of the span (3 or 4, 2),
     contexts end on, before and
     after partition boundaries, and in the ragged bf16 case a 32-row tile of some sequences holds padding rows
-    only (launched without a workspace, in plain order: with one, such batches take the queued launch)."""
+    only (launched without a workspace, in plain order: with one, such batches take the queued launch).  With ALiBi
+    every step goes through the masked variant of the loop, boundaries included."""
     import triton_op_amd as T
 
     gen = torch.Generator().manual_seed(33)
@@ -394,9 +395,10 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
                kv_dtype=kv, scale_mode=scale_mode, block_size=block_size)
     g = wl.to(cuda)
     out = torch.full_like(g.query, float("nan"))
+    slopes = torch.linspace(0.01, 0.3, wl.num_q_heads, dtype=torch.float32) if alibi else None
     plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
                          q_len, 1100, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
-                         query_lens=g.q_lens)
+                         query_lens=g.q_lens, alibi_slopes=None if slopes is None else slopes.to(cuda))
     P = -(-1100 // ps)
     assert plan.args.max_num_partitions == P
     if ragged:
@@ -413,7 +415,7 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     reach = (torch.arange(P)[None, :] * ps < ctx[:, None])  # [batch, P]
     ml, es, to = O.partition_stage(
         wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
-        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, None, ps, P, q_max=wl.q_len)
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, slopes, ps, P, q_max=wl.q_len)
     gml, ges, gto = plan.max_logits.cpu(), plan.exp_sums.cpu(), plan.tmp_output.float().cpu()
     sel = reach[:, None, :, None].expand_as(ml)
     fin = torch.isfinite(ml) & sel
@@ -424,7 +426,7 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     sel_o = reach[:, None, :, None, None].expand_as(to)
     torch.testing.assert_close(gto[sel_o], to[sel_o], atol=ATOL, rtol=RTOL)
     assert not torch.isnan(out.float()).any()
-    torch.testing.assert_close(out.float().cpu(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+    torch.testing.assert_close(out.float().cpu(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
 
 
 @pytest.mark.parametrize("group,q_len,scale_mode", [(8, 1, "tensor"), (16, 3, "token")])

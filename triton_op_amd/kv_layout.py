@@ -9,6 +9,10 @@ Scales: a 0-dim f32 tensor (per tensor) or [num_blocks, num_kv_heads, block_size
 :294-369 (quantize_kv_cache_symmetric), :472-497 (shuffle_value_cache_layout) and
 :792-822 / :903-909 (MTP reshape and its inverse); FP8 here is OCP e4m3fn (max 448), the
 format gfx950 computes in.  Everything is plain torch and runs on CPU or GPU tensors.
+
+The torch quantisers in this file (`quantize_per_tensor`, `pertoken_quant`, `quantize_kv_cache_per_tensor`,
+`quantize_kv_cache_per_token`) build synthetic caches for the workloads and are the formulas the HIP cache
+writers (`kv_cache.py`, `csrc/pa_kv_cache.hip`) are tested against; the writers themselves never call them.
 """
 from __future__ import annotations
 
