@@ -28,7 +28,8 @@ extern "C" {
  * bytes must be zero before the first call; every call leaves the counters (the first 8 bytes) zero, the rest of
  * the 64 bytes is scratch that a call writes before it reads it.  A workspace of
  * pa_decode_workspace_bytes() bytes also has room for the work-item list of the sorted dispatch: in launches of
- * several rounds of workgroups a small planning kernel lists the live (sequence, partition) items, whole
+ * several rounds of workgroups a small planning kernel lists the live (sequence, partition) items (with a small
+ * caller-fixed partition_size: runs of up to four consecutive partitions that one workgroup walks), whole
  * partitions first and the sequences' last, partial partitions by decreasing length, and the partition kernel
  * takes its items from the list (longest-first keeps the end of a ragged batch's launch busy); it also lists the
  * sequences that have more than one partition, which are all that pa_decode's reduce stage then visits.  The
@@ -37,8 +38,10 @@ extern "C" {
 #define PA_DECODE_WORKSPACE_BYTES 64
 /*
  * flags: the workspace still holds the item list that an earlier call built for the SAME context_lens contents,
- * num_seqs, max_num_partitions and partition_size (the previous layer of one decode step, say): the planning
- * kernel is skipped (about 4.5 us).  Ignored by launches that use no item list.
+ * num_seqs, num_kv_heads, q_len, group_size, block_size, max_num_partitions and partition_size (the previous layer
+ * of one decode step, say; the items a launch lists also depend on how many partitions it gives a workgroup, which
+ * follows from those shapes): the planning kernel is skipped (about 4.5 us).  Ignored by launches that use no item
+ * list.
  */
 #define PA_DECODE_FLAG_REUSE_ITEM_LIST 1
 
