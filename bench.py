@@ -266,6 +266,64 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
             "kernel_us_avg": k_us_avg, "kernel_timing": k_timing}
 
 
+def _sample_power(lib, cfg, stream, seconds):
+    """Keeps the configuration's call running back to back for `seconds` and, from the third second on, reads the
+    board's socket power (amd-smi) and shader clock (rocm-smi) once a second in child processes: what the kernels
+    are given to run on once the power management has settled.  Returns None where the tools give nothing."""
+    import re
+    import subprocess
+    import threading
+
+    import torch
+
+    from triton_op_amd import _cabi
+
+    sh = C.c_void_p(stream.cuda_stream)
+    plans, n = cfg.plans, len(cfg.plans)
+    samples = {"socket_power_W": [], "sclk_MHz": []}
+    stop = threading.Event()
+
+    def tool(cmd, pattern):
+        try:
+            out = subprocess.run(cmd, capture_output=True, text=True, timeout=10).stdout
+        except (OSError, subprocess.TimeoutExpired):
+            return None
+        m = re.search(pattern, out)
+        return float(m.group(1)) if m else None
+
+    def sampler():
+        if stop.wait(2.0):
+            return
+        while not stop.is_set():
+            w = tool(["amd-smi", "metric", "-p"], r"SOCKET_POWER:\s*([0-9.]+)\s*W")
+            c = tool(["rocm-smi", "--showclocks"], r"sclk clock level: \d+: \(([0-9.]+)Mhz\)")
+            if w is not None:
+                samples["socket_power_W"].append(w)
+            if c is not None:
+                samples["sclk_MHz"].append(c)
+            stop.wait(1.0)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    t0, calls = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for i in range(200):
+            rc = lib.pa_decode(C.byref(plans[(calls + i) % n].args), sh)
+            if rc:
+                _cabi.check(rc, "pa_decode")
+        calls += 200
+        torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    stop.set()
+    th.join(15.0)
+    cap = tool(["rocm-smi", "--showmaxpower"], r"Max Graphics Package Power \(W\):\s*([0-9.]+)")
+    if not samples["socket_power_W"] and not samples["sclk_MHz"]:
+        return None
+    return {"seconds": round(dt, 1), "calls": calls, "us_per_call_wall": round(dt / calls * 1e6, 2),
+            "socket_power_W": samples["socket_power_W"], "sclk_MHz": samples["sclk_MHz"], "power_cap_W": cap,
+            "how": "amd-smi metric -p and rocm-smi --showclocks, once a second from the third second of a back-to-back loop"}
+
+
 def _traffic(cfg):
     entry = HBM_TRAFFIC.get((cfg.wl0.name, cfg.partition_size))
     if entry is None:
@@ -416,6 +474,8 @@ def _bench_decode(a) -> int:
         result["configs"] = lines
 
     result["roofline"]["device_copy_GBps"] = round(_device_copy_gbps(dev, stream), 1)
+    if a.power_seconds > 0:
+        result["power"] = _sample_power(lib, cfg, stream, a.power_seconds)
     if not a.no_cpu_baseline:
         # a bounded sample: the first sequences of pool 0, copied to the host
         nsamp = min(wl0.batch, 16)
@@ -637,6 +697,8 @@ def main() -> int:
     ap.add_argument("--pools", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="default run: the headline only")
+    ap.add_argument("--power-seconds", type=float, default=0.0,
+                    help="also loop the workload for this long and sample socket power and shader clock (amd-smi, rocm-smi)")
     ap.add_argument("--batch", type=int, default=0, help="override the batch size (debugging only)")
     ap.add_argument("--settle", type=int, default=SETTLE_CALLS,
                     help="untimed calls before anything is measured (profiling runs lower it)")
