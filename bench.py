@@ -464,11 +464,11 @@ def _bench_decode(a) -> int:
         lines = []
         # c2 at the configuration's literal partition size 256 (the reference's constant): same pools
         c2_256 = _Config("c2", dev, a.pools, 256, shared_from=cfg)
-        lines.append(_config_line(c2_256, _time_config(lib, c2_256, stream, min(a.steps, 30), 5, 30)))
+        lines.append(_config_line(c2_256, _time_config(lib, c2_256, stream, min(a.steps, 30), 5, a.settle)))
         del c2_256
         for name in ("c3", "c4", "c5"):
             other = _Config(name, dev, 1)  # each of them streams far more than the last-level cache holds
-            lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 30), 5, 30)))
+            lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 30), 5, a.settle)))
             del other
             torch.cuda.empty_cache()
         result["configs"] = lines
