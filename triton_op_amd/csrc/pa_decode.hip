@@ -205,7 +205,7 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     if (a.block_size > 64 && a.partition_size < 512) span = 1;
     if (forced_span > 0) span = forced_span;
     span = span > a.max_num_partitions ? a.max_num_partitions : span;
-    span = span > 4 ? 4 : span;
+    span = span > kSpanMax ? kSpanMax : span;
     if (span >= 2) {
       c.span = (int)span;
       const long long coarse = (a.max_num_partitions + span - 1) / span;

@@ -68,7 +68,6 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // SPAN: the partial results of the partitions a workgroup has left behind wait here for the end of the pass
   // (stores in the middle of the page stream would hold up the loads issued after them: memory operations of a
   // wave retire in order).  Per partition and row tile: 16 staged bf16 rows, then 16 maxima and 16 sums.
-  constexpr int kSpanMax = 4;
   constexpr int kSpanSlotBytes = 16 * kORowBytes + 2 * 16 * 4;
   constexpr bool kSpanCapable = WAVES == 1 && !QUEUE;
   __shared__ __attribute__((aligned(16))) char span_lds[kSpanCapable ? (kSpanMax - 1) * NT * kSpanSlotBytes : 16];
