@@ -221,16 +221,17 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
     # kernels run in between and every launch gets an event pair of its own (which also brackets its dispatch).
     solo = plans[0].args.max_num_partitions == 1
     if solo:
+        k_launches = max(steps, 100)  # (a short run's 20 launches would mostly measure the first one's ramp)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
-        for i in range(steps):
+        for i in range(k_launches):
             rc = lib.pa_decode_partition(C.byref(plans[i % n].args), sh)
             if rc:
                 _cabi.check(rc, "pa_decode_partition")
         e1.record(stream)
         torch.cuda.synchronize()
-        k_us_avg = e0.elapsed_time(e1) * 1e3 / steps
-        k_timing = f"one event pair around {steps} back-to-back launches"
+        k_us_avg = e0.elapsed_time(e1) * 1e3 / k_launches
+        k_timing = f"one event pair around {k_launches} back-to-back launches"
     else:
         kevs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         for i in range(steps):
