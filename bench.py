@@ -45,6 +45,9 @@ HBM_TRAFFIC = {
     ("c2_fp8_b64_ctx4k", 4096): {
         "bytes": 541_400_000, "launch": "pa_partition_kernel<fp8, bs16, 4 waves> x 512",
         "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
+    ("c2_fp8_b64_ctx4k", 256): {
+        "bytes": 556_600_000, "launch": "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 4 partitions per workgroup",
+        "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
     ("c5_ragged_mix", 7424): {
         "bytes": 2_050_500_000,
         "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items",
