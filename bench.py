@@ -491,6 +491,22 @@ def _bench_decode(a) -> int:
 # ---------------------------------------------------------------------------------------------------------------
 # the read-only probe of c2's gather pattern
 # ---------------------------------------------------------------------------------------------------------------
+def _load_probe_library():
+    """libpa_probe.so: the two measuring kernels (tests/native/pa_probe.h), a library of their own beside the
+    operator's; built by `python -m triton_op_amd.build`."""
+    from triton_op_amd import _cabi
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "native", "libpa_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python -m triton_op_amd.build`")
+    lib = C.CDLL(path)
+    lib.pa_probe_gather.restype = C.c_int
+    lib.pa_probe_gather.argtypes = [C.POINTER(_cabi.PaDecodeArgs), C.c_void_p, C.c_void_p]
+    lib.pa_probe_issue.restype = C.c_int
+    lib.pa_probe_issue.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
+    return lib
+
+
 def _bench_probe_gather(a) -> int:
     """Reads exactly the pages c2's partition kernel reads, in the same order and grouping (one workgroup of four
     waves per (sequence, kv head), each wave every fourth 64-token step, 16 bytes per lane, non-temporal), and does
@@ -502,7 +518,7 @@ def _bench_probe_gather(a) -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
-    lib = _cabi.load_library()
+    lib = _load_probe_library()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream(dev)
@@ -511,9 +527,9 @@ def _bench_probe_gather(a) -> int:
     sink = torch.zeros(64, dtype=torch.int32, device=dev)
 
     def call(i):
-        rc = lib.pa_debug_gather_probe(C.byref(cfg.plans[i % len(cfg.plans)].args), C.c_void_p(sink.data_ptr()), sh)
+        rc = lib.pa_probe_gather(C.byref(cfg.plans[i % len(cfg.plans)].args), C.c_void_p(sink.data_ptr()), sh)
         if rc:
-            _cabi.check(rc, "pa_debug_gather_probe")
+            _cabi.check(rc, "pa_probe_gather")
 
     for i in range(a.settle):
         call(i)
@@ -539,7 +555,7 @@ def _bench_probe_gather(a) -> int:
 
 
 def _bench_probe_issue(a) -> int:
-    """What the instructions of the decode step cost a SIMD's issue port (pa_debug_issue_probe): nanoseconds per
+    """What the instructions of the decode step cost a SIMD's issue port (pa_probe_issue): nanoseconds per
     instruction per wave with one and with three waves on every SIMD, and how far the matrix pipe runs beside the
     vector ALU."""
     import torch
@@ -549,7 +565,7 @@ def _bench_probe_issue(a) -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
-    lib = _cabi.load_library()
+    lib = _load_probe_library()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream(dev)
@@ -564,7 +580,7 @@ def _bench_probe_issue(a) -> int:
     for mode in range(6):
         for waves in (1, 3):
             def call():
-                _cabi.check(lib.pa_debug_issue_probe(mode, iters, cus * waves, C.c_void_p(sink.data_ptr()), sh), "probe")
+                _cabi.check(lib.pa_probe_issue(mode, iters, cus * waves, C.c_void_p(sink.data_ptr()), sh), "probe")
             call()
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

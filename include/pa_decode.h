@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define PA_DECODE_ABI_VERSION 4
+#define PA_DECODE_ABI_VERSION 5
 /* Smallest useful size of the optional device workspace.  Its first 64 bytes hold a work-item counter: with
  * it, batches with per-sequence query lengths are launched as a resident grid that pulls live (sequence,
  * partition, row tile, head) items from the counter instead of one workgroup per possible item.  These 64
@@ -98,9 +98,10 @@ typedef struct PaDecodeArgs {
   const float* query_scale;   /* optional; per tensor: 1 value, per token: [B, Hkv*Ge, 1] */
   const float* key_scale;     /* optional */
   const float* value_scale;   /* optional */
-  const float* alibi_slopes;  /* optional, [Hkv*G]: one slope per query HEAD, shared by the q new tokens of a head (the
-                                 reference kernel indexes [Hkv*q*G] like sinks, pa_decode_triton_gluon_fp8.py:323-327;
-                                 the two agree for q_len == 1) */
+  const float* alibi_slopes;  /* optional, alibi_slopes_len f32 values: one slope per packed query ROW, [Hkv*q*G] at
+                                 h*Ge + t*G + g, as the reference kernels index it (pa_decode_triton_gluon_fp8.py:323-327,
+                                 803-810: alibi_slopes_ptr + kv_head*QUERY_GROUP_SIZE + row), or one per query HEAD,
+                                 [Hkv*G] at h*G + g, shared by the q new tokens of a head; the same array for q_len == 1 */
   const float* sinks;         /* optional, [Hkv*Ge]: attention-sink logit of every query row (natural-log domain) */
   float* exp_sums;
   float* max_logits;
@@ -122,6 +123,10 @@ typedef struct PaDecodeArgs {
   int32_t query_quant_mode;    /* PA_QUANT_* */
   int32_t kv_quant_mode;       /* PA_QUANT_* */
   int32_t v_transposed;
+  int32_t alibi_slopes_len;    /* elements of alibi_slopes: num_kv_heads*q_len*group_size (per row) or
+                                  num_kv_heads*group_size (per head); anything else is PA_ERR_BAD_SHAPE; ignored
+                                  when alibi_slopes is NULL */
+  int32_t reserved0;           /* 0 */
   float softmax_scale;
 
   int64_t stride_out_s, stride_out_h;
@@ -194,8 +199,8 @@ int pa_decode(const PaDecodeArgs* args, void* hip_stream);
  * sequences; the sorted dispatch's planning kernel takes at most 4096.
  *
  * Environment: none of the library's behaviour depends on environment variables unless the process was started
- * with PA_DECODE_DEBUG=1, which enables the tuning switches PA_DECODE_WAVES, PA_DECODE_QUEUE, PA_DECODE_SHARED
- * and PA_DECODE_SORTED (read once, at the first launch).
+ * with PA_DECODE_DEBUG=1, which enables the tuning switches PA_DECODE_WAVES, PA_DECODE_ROW_TILES, PA_DECODE_SPAN,
+ * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED and PA_DECODE_LDS_PAD (read once, at the first launch).
  */
 int pa_decode_launch_info(const PaDecodeArgs* args, char* text, int32_t text_bytes);
 
@@ -270,25 +275,6 @@ int pa_quantize_kv_cache(const void* key_cache_bf16, const void* value_cache_bf1
  * with the format definition code by code.
  */
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream);
-
-/*
- * Measurement hook: a read-only probe of the memory access pattern of stage 1.  For the same arguments it reads
- * the K and V bytes that the partition kernel for up to 16 query rows reads (FP8 cache, block size 16, dense
- * layout; anything else is PA_ERR_UNSUPPORTED), with the same workgroup decomposition, load width and cache
- * policy, and does no arithmetic: its duration is what the memory system gives the gather pattern.  sink: at
- * least 64 int32 of device memory (written only in a case that does not occur; it keeps the loads alive).
- */
-int pa_debug_gather_probe(const PaDecodeArgs* args, int32_t* sink, void* hip_stream);
-
-/*
- * Measurement hook: the issue cost of the instructions the decode step is made of.  Launches `workgroups` workgroups
- * of four waves (one per SIMD; 256 x n workgroups put n waves on every SIMD of a 256-CU GPU) that each run
- * `iterations` x 128 instructions of one kind: mode 0 v_fma_f32 (the full-rate yardstick), 3 v_exp_f32,
- * 4 v_cvt_pk_fp8_f32, 5 v_permlane32_swap; mode 1 runs iterations x 16 v_mfma_f32_16x16x128_f8f6f4, mode 2 the same
- * 16 MFMAs with eight independent v_fma_f32 behind each (how far the matrix pipe runs beside the vector ALU).
- * sink: at least 64 int32 of device memory (not written in practice).  Time it with events on the stream.
- */
-int pa_debug_issue_probe(int32_t mode, int32_t iterations, int32_t workgroups, int32_t* sink, void* hip_stream);
 
 #ifdef __cplusplus
 }

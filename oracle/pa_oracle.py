@@ -27,6 +27,9 @@ un-installed ``aiter`` package and a gfx942 GPU):
   - causal MTP mask   by exhaustive enumeration against tril(diagonal=key_len-query_len)
   - partition/reduce  by independence of the result from the partition size, by the
                       one-partition identity, and by the closed-form log-sum-exp merge
+  - ALiBi             by an explicit per-row bias matrix added to a dense softmax (one slope per packed row,
+                      several new tokens and kv heads, all slopes different; swapping two rows' slopes must
+                      move exactly those rows), and per-head slopes by equality with their per-row expansion
 The reference holds no golden vectors or known-answer tests for this path (its logs keep only
 md5s of GPU-RNG outputs in fnuz FP8); bit-exact agreement with the reference's *kernels*
 (accumulation order, exp2 implementation, P->FP8 rounding) is therefore "parity unpinned";
@@ -157,7 +160,7 @@ def masked_attention(
     softmax_scale: float,
     output_dtype: torch.dtype,
     is_causal: bool = True,
-    alibi_slopes: Optional[torch.Tensor] = None,  # [Hq]
+    alibi_slopes: Optional[torch.Tensor] = None,  # [Hq] (shared by the q new tokens), or [q, Hq]: one per query row
     sinks: Optional[torch.Tensor] = None,  # [q, Hq] attention-sink logits
 ) -> torch.Tensor:
     hq, hkv = query.shape[1], key.shape[1]
@@ -166,9 +169,12 @@ def masked_attention(
     scores = torch.einsum("qhd,khd->hqk", query.float(), key.float()) * softmax_scale
     qlen, klen = query.shape[0], key.shape[0]
     if alibi_slopes is not None:
-        # pa_decode_triton_gluon_fp8.py:906-908: slope * (col - ctx + 1), same for every new token
+        # pa_decode_triton_gluon_fp8.py:906-908: slope_of_row * (col - ctx + 1); the column offset is the same for
+        # every new token, the slope is read per packed query row (:323-327, :803-810)
         pos = torch.arange(klen, dtype=torch.float32) - klen + 1
-        scores = scores + alibi_slopes.float()[:, None, None] * pos[None, None, :]
+        sl = alibi_slopes.float()
+        sl = sl[:, None].expand(hq, qlen) if sl.dim() == 1 else sl.t()  # [Hq, q]
+        scores = scores + sl[:, :, None] * pos[None, None, :]
     if is_causal:
         bias = torch.zeros(qlen, klen, dtype=torch.float32)
         keep = torch.ones(qlen, klen, dtype=torch.bool).tril(diagonal=klen - qlen)
@@ -224,6 +230,20 @@ def mha_extend(
     return out
 
 
+def _alibi_of_rows(alibi_slopes: Optional[torch.Tensor], hkv: int, qmax: int, g: int) -> Optional[torch.Tensor]:
+    """ALiBi slopes of the packed query rows, [Hkv, qmax, G].  The entry point takes one slope per packed row,
+    [Hkv*qmax*G] at h*(qmax*G) + t*G + g -- the array the reference kernels index with
+    kv_head*QUERY_GROUP_SIZE + row (pa_decode_triton_gluon_fp8.py:323-327, 803-810) -- or one per query head,
+    [Hkv*G], shared by the head's new tokens; for one new token the two are the same array."""
+    if alibi_slopes is None:
+        return None
+    sl = alibi_slopes.float().reshape(-1)
+    if sl.numel() == hkv * qmax * g:
+        return sl.view(hkv, qmax, g)
+    assert sl.numel() == hkv * g, (sl.numel(), hkv, qmax, g)
+    return sl.view(hkv, 1, g).expand(hkv, qmax, g)
+
+
 def _row_qlens(batch: int, qlen: Union[int, torch.Tensor, Sequence[int]], q_max: Optional[int] = None):
     """per-sequence query lengths and the number of query positions the packed rows are laid out for"""
     if isinstance(qlen, int):
@@ -271,10 +291,12 @@ def paged_attention_decode_oracle(
         k, v = gather_sequence(key_flat, value_flat, ks, vs, block_tables[b], ctx, bs)
         # [Hkv, qmax, G, D] -> token-major [qb, Hq, D]
         qv = qf[b].view(hkv, qmax, g, d)[:, :qb].permute(1, 0, 2, 3).reshape(qb, hkv * g, d)
-        sk = None
+        sk = al = None
         if sinks is not None:
             sk = sinks.float().view(hkv, qmax, g)[:, :qb].permute(1, 0, 2).reshape(qb, hkv * g)
-        o = masked_attention(qv, k, v, softmax_scale, torch.float32, True, alibi_slopes, sk)
+        if alibi_slopes is not None:  # token-major like the query: [qb, Hq]
+            al = _alibi_of_rows(alibi_slopes, hkv, qmax, g)[:, :qb].permute(1, 0, 2).reshape(qb, hkv * g)
+        o = masked_attention(qv, k, v, softmax_scale, torch.float32, True, al, sk)
         o = o.view(qb, hkv, g, d).permute(1, 0, 2, 3)  # [Hkv, qb, G, D]
         out[b].view(hkv, qmax, g, d)[:, :qb] = o.to(out_dtype)
     return out
@@ -332,7 +354,7 @@ def partition_stage(
         scores = torch.einsum("hrd,khd->hrk", qv, k) * softmax_scale  # [Hkv, Ge, ctx]
         col = torch.arange(ctx)
         if alibi_slopes is not None:
-            sl = alibi_slopes.float().view(hkv, 1, g).expand(hkv, qmax, g).reshape(hkv, ge)
+            sl = _alibi_of_rows(alibi_slopes, hkv, qmax, g).reshape(hkv, ge)
             scores = scores + sl[:, :, None] * (col - ctx + 1).float()[None, None, :]
         t_of_row = torch.arange(ge) // g
         # visible: col + (q-1-t) < ctx   (pa_decode_triton_gluon_fp8.py:917-918); padded t masked

@@ -2,7 +2,7 @@
 #ifndef PA_PROBE_KERNEL_H_
 #define PA_PROBE_KERNEL_H_
 
-#include "pa_common.h"
+#include "../../triton_op_amd/csrc/pa_common.h"
 
 namespace {
 

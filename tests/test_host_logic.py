@@ -131,6 +131,53 @@ def test_entry_point_rejects_bad_arguments(over, msg):
         T.plan_decode(**_cpu_args(**over))
 
 
+def test_entry_point_takes_the_harness_wrappers_trailing_buffers_and_both_alibi_layouts():
+    """`max_logits, exp_sums, tmp_output` follow `alibi_slopes` positionally, as in run_gluon_fp8_kernel
+    (test_pa_mtp.py:566-584; its spelling `temp_output` is a keyword here) and run_triton
+    (test_pa_decode_gluon_triton.py:264-281); `alibi_slopes` is one slope per packed query row (the reference
+    kernels' array, pa_decode_triton_gluon_fp8.py:323-327) or one per query head.  On this GPU-less machine a call
+    that passes every argument check ends at the "GPU only" error; anything else raised earlier."""
+    from triton_op_amd import pa_decode_triton
+
+    wl = W.make_decode_workload(name="v", seed=1, batch=2, num_q_heads=8, num_kv_heads=2, q_len=3,
+                                context_lens=torch.tensor([40, 300], dtype=torch.int32))
+    rows = 2 * 3 * 4
+    ml, es = torch.zeros(2, 2, 2, 12), torch.zeros(2, 2, 2, 12)
+    to = torch.zeros(2, 2, 2, 12, 128, dtype=torch.bfloat16)
+    pos = (torch.empty_like(wl.query), wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+           wl.softmax_scale, 3, 300, torch.bfloat16, None, wl.key_scale, wl.value_scale, 0)
+    for slopes in (torch.rand(rows), torch.rand(8), None):
+        with pytest.raises(ValueError, match="GPU only"):
+            T.plan_decode(*pos, slopes, ml, es, to)
+        with pytest.raises(ValueError, match="GPU only"):
+            T.paged_attention_decode(*pos, slopes, ml, es, temp_output=to)
+    for bad in (torch.rand(rows + 1), torch.rand(2), torch.rand(rows, dtype=torch.float64)):
+        with pytest.raises(ValueError, match="alibi_slopes must be"):
+            T.plan_decode(*pos, bad)
+    with pytest.raises(ValueError, match="same buffer"):
+        T.plan_decode(*pos, None, ml, es, to, temp_output=to.clone())
+    wl1 = W.make_decode_workload(name="v", seed=1, batch=2, num_q_heads=8, num_kv_heads=2,
+                                 context_lens=torch.tensor([40, 300], dtype=torch.int32))
+    with pytest.raises(ValueError, match="GPU only"):
+        pa_decode_triton.paged_attention_decode(
+            torch.empty_like(wl1.query), wl1.query, wl1.key_cache, wl1.value_cache, wl1.context_lens, wl1.block_tables,
+            wl1.softmax_scale, 300, torch.bfloat16, wl1.key_scale, wl1.value_scale, 0, torch.rand(8),
+            torch.zeros(2, 2, 2, 4), torch.zeros(2, 2, 2, 4), torch.zeros(2, 2, 2, 4, 128, dtype=torch.bfloat16))
+
+
+def test_c_abi_checks_the_alibi_array_length(pa_lib):
+    """The C ABI cannot see an array's length: alibi_slopes_len says which of the two layouts the caller's array
+    has, and anything else is refused before a launch."""
+    a = _fake_args(b=4, hq=16, hkv=2, q=3, ctx=1024, ps=256)
+    buf = C.create_string_buffer(256)
+    a.alibi_slopes = 0x70000000
+    for n, rc in ((2 * 3 * 8, 0), (2 * 8, 0), (0, -4), (3 * 8, -4), (2 * 3 * 8 + 1, -4)):
+        a.alibi_slopes_len = n
+        assert pa_lib.pa_decode_launch_info(C.byref(a), buf, 256) == rc, n
+    a.alibi_slopes = None  # without slopes the length is ignored
+    assert pa_lib.pa_decode_launch_info(C.byref(a), buf, 256) == 0
+
+
 def test_entry_point_rejects_group_and_block_size():
     wl = W.make_decode_workload(name="v", seed=1, batch=1, num_q_heads=80, num_kv_heads=1,
                                 context_lens=torch.tensor([40], dtype=torch.int32))

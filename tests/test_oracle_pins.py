@@ -317,3 +317,46 @@ def test_error_stats_on_a_hand_computed_pair():
     assert st["nan_result"] == 0 and st["nan_ref"] == 0
     st = O.error_stats(torch.tensor([float("nan"), 1.0]), torch.tensor([0.0, 1.0]))
     assert st["nan_result"] == 1 and st["nan_ref"] == 0
+
+
+def test_alibi_per_packed_row_matches_explicit_bias():
+    """One ALiBi slope per PACKED query row, [Hkv*q*G] at h*q*G + t*G + g: what the reference kernels read with
+    alibi_slopes_ptr + kv_head*QUERY_GROUP_SIZE + row (pa_decode_triton_gluon_fp8.py:323-327, 803-810) and add as
+    slope[row] * (col - ctx + 1) (:906-908).  Three new tokens, two kv heads, all slopes different; every row is
+    held against a dense softmax with the bias written out as a matrix.  A slope array read in (t, h, g) or
+    (h, g, t) order pairs rows with other rows' slopes and fails; so does a bias that counts columns from the
+    row's own last visible key instead of from the context's end."""
+    q_len, hq, hkv = 3, 4, 2
+    g = hq // hkv
+    wl = _tiny("bf16", "none", q_len=q_len, hq=hq, hkv=hkv, ctx=(9, 21, 40))
+    rows = hkv * q_len * g
+    slopes = torch.linspace(0.02, 0.9, rows)  # one per packed row, all different
+    out = _oracle(wl, alibi_slopes=slopes)
+    kf, vf = O.flatten_key_cache(wl.key_cache), O.flatten_value_cache(wl.value_cache)
+    for b, ctx in enumerate((9, 21, 40)):
+        k, v = O.gather_sequence(kf, vf, None, None, wl.block_tables[b], ctx, 16)  # [ctx, Hkv, D]
+        bias = slopes.double()[:, None] * (torch.arange(ctx) - ctx + 1).double()[None, :]  # [rows, ctx]
+        for h in range(hkv):
+            for t in range(q_len):
+                for gg in range(g):
+                    row = h * q_len * g + t * g + gg
+                    nvis = ctx - (q_len - 1 - t)
+                    s = (k[:nvis, h].double() @ wl.query[b, row].double()) * wl.softmax_scale + bias[row, :nvis]
+                    o = torch.softmax(s, 0) @ v[:nvis, h].double()
+                    torch.testing.assert_close(out[b, row].double(), o.to(torch.bfloat16).double(), atol=1e-2, rtol=1e-2)
+    # swapping the slopes of two rows moves exactly those rows
+    sw = slopes.clone()
+    sw[[1, 8]] = slopes[[8, 1]]
+    moved = _oracle(wl, alibi_slopes=sw)
+    same = [r for r in range(rows) if r not in (1, 8)]
+    assert torch.equal(moved[:, same], out[:, same])
+    assert not torch.equal(moved[:, 1], out[:, 1]) and not torch.equal(moved[:, 8], out[:, 8])
+    # one slope per query head is the per-row array with the head's slope repeated for its new tokens
+    per_head = torch.tensor([0.5, 0.25, 0.125, 0.0625])
+    expanded = per_head.view(hkv, 1, g).expand(hkv, q_len, g).reshape(-1)
+    assert torch.equal(_oracle(wl, alibi_slopes=per_head), _oracle(wl, alibi_slopes=expanded))
+    # and the two-stage form reads the same array the same way
+    ml, es, to = O.partition_stage(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                   wl.softmax_scale, q_len, wl.key_scale, wl.value_scale, slopes, 256)
+    merged = O.reduce_stage(ml, es, to, wl.context_lens, 256)
+    torch.testing.assert_close(merged.float(), out.float(), atol=2e-3, rtol=2 ** -7)

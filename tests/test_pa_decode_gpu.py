@@ -135,6 +135,10 @@ CASES = {
     "fp8_token_ragged_two_waves_per_tile": dict(batch=5, num_q_heads=32, num_kv_heads=2,
                                                 context_lens=_ctx(17, 64, 1000, 2, 300), q_len=4,
                                                 q_lens=_ctx(2, 1, 2, 2, 1), scale_mode="token"),
+    # a bf16 cache with 64 rows per kv head and ragged query lengths: two workgroups of two row tiles per kv head,
+    # taken from the work queue when the call has a workspace (tiles of padding rows only are no items)
+    "bf16_ragged_g16_q4": dict(batch=5, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(300, 33, 700, 4, 257), q_len=4,
+                               q_lens=_ctx(1, 4, 2, 3, 4), kv_dtype="bf16", scale_mode="none"),
     "bf16_transV_bs64": dict(batch=2, num_q_heads=8, num_kv_heads=2, context_lens=_ctx(150, 300), block_size=64,
                              kv_dtype="bf16", scale_mode="none", transposed_v=True),
 }
@@ -156,13 +160,23 @@ def test_parity_stagewise_and_end_to_end(cuda, name, partition_size):
     assert thr < 1e-2, thr
 
 
-@pytest.mark.parametrize("name", ["fp8_g8", "fp8_g10_q3", "fp8_token_g16_q4"])
-def test_alibi(cuda, name):
+@pytest.mark.parametrize("name", ["fp8_g8", "fp8_g10_q3", "fp8_token_g16_q4", "bf16_g16_q4", "fp8_token_ragged"])
+@pytest.mark.parametrize("layout", ["per_row", "per_head"])
+def test_alibi(cuda, name, layout):
+    """ALiBi slopes in both layouts the entry point takes: one per packed query row, [Hkv*q*G] -- the array the
+    reference kernels index with kv_head*QUERY_GROUP_SIZE + row (pa_decode_triton_gluon_fp8.py:323-327, 803-810) --
+    and one per query head.  With several new tokens the per-row slopes are all different, so a kernel that read
+    them per head (or in another row order) misses the oracle."""
     wl = _make(**CASES[name])
-    slopes = torch.linspace(0.01, 0.3, wl.num_q_heads, dtype=torch.float32)
+    n = wl.query.shape[1] if layout == "per_row" else wl.num_q_heads
+    slopes = torch.linspace(0.01, 0.3, n, dtype=torch.float32)
     out, res = _run(wl, cuda, alibi=slopes)
-    torch.testing.assert_close(out.float(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
+    ref = _oracle(wl, slopes)
+    torch.testing.assert_close(out.float(), ref.float(), atol=ATOL, rtol=RTOL)
     _check_stages(wl, res, 256, slopes)
+    if layout == "per_row" and wl.q_len > 1:  # the other reading of the same numbers is a different result
+        other = _oracle(wl, slopes[:wl.num_q_heads])
+        assert float((other.float() - ref.float()).abs().max()) > 5e-2
 
 
 @pytest.mark.parametrize("q_len", [2, 4])
@@ -341,9 +355,13 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     import triton_op_amd as T
 
     gen = torch.Generator().manual_seed(21)
-    batch = 96
-    ctx = torch.randint(1, 2600, (batch,), generator=gen, dtype=torch.int32)
-    ctx[:5] = torch.tensor([512, 256, 2560, 1, 255], dtype=torch.int32)
+    # one row tile per kv head: one-wave workgroups walk up to four partitions each, so it takes 600 sequences
+    # before the coarser items still make more than two rounds (600 x 8 x ceil(5 / 4)); the shared-stream kernel
+    # (48 rows) has one item per partition and 96 sequences are plenty
+    batch = 96 if group * q_len > 16 else 600
+    top = 2600 if group * q_len > 16 else 1280
+    ctx = torch.randint(1, top, (batch,), generator=gen, dtype=torch.int32)
+    ctx[:5] = torch.tensor([512, 256, top - 40, 1, 255], dtype=torch.int32)
     ctx = torch.clamp(ctx, min=q_len)
     wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, scale_mode=scale_mode)
     g = wl.to(cuda)
@@ -358,6 +376,10 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
                              g.softmax_scale, q_len, g.max_context_len, torch.bfloat16, None, g.key_scale,
                              g.value_scale, partition_size=256, workspace=ws)
         assert plan.args.max_num_partitions * batch * 8 > 4096  # far more workgroups than the GPU holds
+        info = plan.launch_info()
+        print(f"workspace {ws_bytes}: {info}", flush=True)
+        # the first two launches really take their items from the list, the third really does not
+        assert ("sorted items" in info) == (ws_bytes != 64), info
         plan.run()
         plan.run()  # the list is rebuilt by every call
         torch.cuda.synchronize()
@@ -367,11 +389,13 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
-@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span,alibi",
-                         [("fp8", "tensor", 2, 1, False, 16, 256, 3, False), ("fp8", "token", 4, 2, False, 16, 256, 3, False),
-                          ("fp8", "tensor", 8, 2, False, 64, 256, 3, False), ("fp8", "tensor", 8, 2, False, 1024, 512, 2, False),
-                          ("bf16", "none", 16, 4, True, 16, 256, 4, False), ("fp8", "token", 8, 1, False, 16, 256, 3, True)])
-def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span, alibi):
+@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span,alibi,batch",
+                         [("fp8", "tensor", 2, 1, False, 16, 256, 3, False, 200), ("fp8", "token", 4, 2, False, 16, 256, 3, False, 200),
+                          ("fp8", "tensor", 8, 2, False, 64, 256, 3, False, 200), ("fp8", "tensor", 8, 2, False, 1024, 512, 2, False, 200),
+                          ("bf16", "none", 16, 4, True, 16, 256, 4, False, 200), ("fp8", "token", 8, 1, False, 16, 256, 3, True, 200),
+                          # 600 x 8 x ceil(5 / 4) coarse items are more than two rounds: the walk AND the sorted dispatch
+                          ("fp8", "tensor", 8, 1, False, 16, 256, 4, False, 600), ("fp8", "token", 4, 2, False, 16, 256, 4, True, 600)])
+def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span, alibi, batch):
     """A caller-fixed small partition size and several rounds of one-wave workgroups: every workgroup then walks
     several consecutive partitions in one pass over the pages (the launch layer says so) and writes one partial
     result per partition.  The partition buffers are held against the oracle's partition stage, the merged result
@@ -379,11 +403,14 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     contexts end on, before and
     after partition boundaries, and in the ragged bf16 case a 32-row tile of some sequences holds padding rows
     only (launched without a workspace, in plain order: with one, such batches take the queued launch).  With ALiBi
-    every step goes through the masked variant of the loop, boundaries included."""
+    every step goes through the masked variant of the loop, boundaries included.  The two cases of 600 sequences
+    still have more than two rounds of the coarser items, so the planning kernel lists (sequence, first partition of
+    a walk) items and the workgroups take them from the list: there one sequence is empty, and the call is made a
+    second time with the flag that says the list is still good."""
     import triton_op_amd as T
+    from triton_op_amd import _cabi
 
     gen = torch.Generator().manual_seed(33)
-    batch = 200
     ctx = torch.randint(1, 1101, (batch,), generator=gen, dtype=torch.int32)
     ctx[:9] = torch.tensor([1, 255, 256, 257, 512, 768, 769, 1024, 1100], dtype=torch.int32)
     ctx = torch.clamp(ctx, min=q_len)
@@ -393,9 +420,15 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
         q_lens[:4] = torch.tensor([1, q_len, 2, 1], dtype=torch.int32)
     wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, q_lens=q_lens,
                kv_dtype=kv, scale_mode=scale_mode, block_size=block_size)
+    sorted_too = batch == 600
+    if sorted_too:  # an empty sequence among them (the generator wants a page per sequence: declared empty afterwards)
+        ctx = ctx.clone()
+        ctx[11] = 0
+        wl = type(wl)(**{**wl.__dict__, "context_lens": ctx})
+    live = [b for b in range(batch) if int(ctx[b]) > 0]
     g = wl.to(cuda)
     out = torch.full_like(g.query, float("nan"))
-    slopes = torch.linspace(0.01, 0.3, wl.num_q_heads, dtype=torch.float32) if alibi else None
+    slopes = torch.linspace(0.01, 0.3, wl.query.shape[1], dtype=torch.float32) if alibi else None
     plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
                          q_len, 1100, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
                          query_lens=g.q_lens, alibi_slopes=None if slopes is None else slopes.to(cuda))
@@ -407,10 +440,22 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     # 8000 items for 2048 wave slots: three partitions each (4800 of 512 tokens: two); 16000 two-tile items for 1024
     # slots: four, the most there is
     assert f"{span} partitions per workgroup" in plan.launch_info(), plan.launch_info()
+    assert ("sorted items" in plan.launch_info()) == sorted_too, plan.launch_info()
     plan.exp_sums.fill_(float("nan"))
     plan.max_logits.fill_(float("nan"))
     plan.run()
     torch.cuda.synchronize()
+    if sorted_too:
+        # the next layer of the same step: same lengths, the list of coarse items is reused
+        first = out.clone()
+        out.fill_(float("nan"))
+        plan.exp_sums.fill_(float("nan"))
+        plan.max_logits.fill_(float("nan"))
+        plan.args.flags = _cabi.PA_DECODE_FLAG_REUSE_ITEM_LIST
+        plan.run()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), first.view(torch.int16))
+        assert bool((out[11] == 0).all())
     # partitions a sequence does not reach are not written; the oracle leaves them at its fill values
     reach = (torch.arange(P)[None, :] * ps < ctx[:, None])  # [batch, P]
     ml, es, to = O.partition_stage(
@@ -426,7 +471,7 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     sel_o = reach[:, None, :, None, None].expand_as(to)
     torch.testing.assert_close(gto[sel_o], to[sel_o], atol=ATOL, rtol=RTOL)
     assert not torch.isnan(out.float()).any()
-    torch.testing.assert_close(out.float().cpu(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
+    torch.testing.assert_close(out.float().cpu()[live], _oracle(wl, slopes, seq_ids=live).float()[live], atol=ATOL, rtol=RTOL)
 
 
 @pytest.mark.parametrize("group,q_len,scale_mode", [(8, 1, "tensor"), (16, 3, "token")])
@@ -437,8 +482,10 @@ def test_item_list_reused_by_the_next_layer(cuda, group, q_len, scale_mode):
     from triton_op_amd import _cabi
 
     gen = torch.Generator().manual_seed(23)
-    batch = 96
-    ctx = torch.clamp(torch.randint(1, 2600, (batch,), generator=gen, dtype=torch.int32), min=q_len)
+    # (one row tile per kv head: workgroups walk four partitions each, and it takes 600 sequences for the coarser
+    # items to still be listed)
+    batch = 96 if group * q_len > 16 else 600
+    ctx = torch.clamp(torch.randint(1, 2600 if batch == 96 else 1280, (batch,), generator=gen, dtype=torch.int32), min=q_len)
     kw = dict(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, scale_mode=scale_mode)
     layers = [_make(**kw, seed=7).to(cuda), _make(**kw, seed=8).to(cuda)]
     parts = -(-int(ctx.max()) // 256)
@@ -446,9 +493,11 @@ def test_item_list_reused_by_the_next_layer(cuda, group, q_len, scale_mode):
     outs = []
     for i, g in enumerate(layers):
         out = torch.full_like(g.query, float("nan"))
-        T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
-                                 q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
-                                 partition_size=256, workspace=ws, reuse_item_list=i > 0)
+        plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                             q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                             partition_size=256, workspace=ws, reuse_item_list=i > 0)
+        assert "sorted items" in plan.launch_info(), plan.launch_info()
+        plan.run()
         outs.append(out)
     alone = torch.full_like(layers[1].query, float("nan"))
     g = layers[1]
@@ -473,10 +522,11 @@ def test_empty_sequences_get_zero_rows(cuda, case):
         one_partition=(dict(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(100, 0, 200, 0)), 256),
         partitions=(dict(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(700, 0, 200, 0)), 256),
         shared=(dict(batch=4, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(100, 0, 200, 0), q_len=3), 256),
-        sorted=(dict(batch=96, num_q_heads=16, num_kv_heads=8,
-                     context_lens=torch.cat([_ctx(0, 1500, 0), torch.randint(1, 2600, (93,),
+        sorted=(dict(batch=600, num_q_heads=16, num_kv_heads=8,
+                     context_lens=torch.cat([_ctx(0, 1100, 0), torch.randint(1, 1280, (597,),
                                             generator=torch.Generator().manual_seed(5), dtype=torch.int32)])), 256),
-        queue=(dict(batch=4, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 0, 200, 0), q_len=4,
+        # (a bf16 cache takes two 16-row tiles per workgroup: the queued launch needs more than 32 rows per kv head)
+        queue=(dict(batch=4, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(300, 0, 200, 0), q_len=4,
                     q_lens=_ctx(4, 2, 1, 4), kv_dtype="bf16", scale_mode="none"), 512),
     )[case]
     # the generator wants at least one page per sequence: build with length 1, then declare the sequences empty
@@ -486,6 +536,12 @@ def test_empty_sequences_get_zero_rows(cuda, case):
     ctx[empty] = 0
     wl = type(wl)(**{**wl.__dict__, "context_lens": ctx})
     out, _ = _run(wl, cuda, partition_size=ps)
+    if case in ("sorted", "queue"):  # the launch mode the case is named for is the one that ran
+        g = wl.to(cuda)
+        info = T.plan_decode(torch.empty_like(g.query), g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                             g.softmax_scale, g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                             partition_size=ps, query_lens=g.q_lens).launch_info()
+        assert ("sorted items" if case == "sorted" else "queued items") in info, info
     assert not torch.isnan(out.float()).any()
     assert bool((out[empty] == 0).all())
     live = [i for i in range(len(ctx)) if not bool(empty[i])]
@@ -516,11 +572,13 @@ def test_graph_capture_and_replay(cuda, case):
     import triton_op_amd as T
 
     gen = torch.Generator().manual_seed(31)
-    if case == "queue":  # bf16 cache, 32 query rows, ragged query lengths: the queued launch
-        kw = dict(batch=6, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000, 17, 700, 256), q_len=4,
+    if case == "queue":  # bf16 cache, 64 query rows (two workgroups of two row tiles), ragged query lengths: the queued launch
+        kw = dict(batch=6, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(300, 64, 1000, 17, 700, 256), q_len=4,
                   q_lens=_ctx(1, 4, 2, 3, 4, 1), kv_dtype="bf16", scale_mode="none")
     elif case == "sorted":  # several rounds of workgroups: the planning kernel runs inside the graph
-        kw = dict(batch=96, num_q_heads=32, num_kv_heads=8, q_len=2,
+        # (32 rows per kv head: one item per partition; with up to 16 rows the workgroups would walk four
+        # partitions each and 96 sequences would be a single round)
+        kw = dict(batch=96, num_q_heads=128, num_kv_heads=8, q_len=2,
                   context_lens=torch.randint(2, 2600, (96,), generator=gen, dtype=torch.int32))
     else:
         kw = dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000))
@@ -530,6 +588,8 @@ def test_graph_capture_and_replay(cuda, case):
     plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
                          g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
                          partition_size=256, query_lens=g.q_lens)
+    if case != "plain":  # the launch mode the case is named for is the one that is captured
+        assert ("queued items" if case == "queue" else "sorted items") in plan.launch_info(), plan.launch_info()
     plan.run()
     torch.cuda.synchronize()
     eager = out.clone()
@@ -636,7 +696,8 @@ def test_seeded_random_sweep(cuda, seed):
     print(f"seed={seed} ps={ps} alibi={alibi} " + " ".join(f"{k}={v.tolist() if torch.is_tensor(v) else v}" for k, v in kw.items()),
           flush=True)
     wl = _make(**kw)
-    slopes = torch.linspace(0.02, 0.4, wl.num_q_heads, dtype=torch.float32) if alibi else None
+    # odd seeds: one slope per packed query row (the reference kernels' array), even seeds: one per query head
+    slopes = torch.linspace(0.02, 0.4, wl.query.shape[1] if seed % 2 else wl.num_q_heads, dtype=torch.float32) if alibi else None
     out, res = _run(wl, cuda, partition_size=ps, alibi=slopes)
     assert not torch.isnan(out.float()).any()
     torch.testing.assert_close(out.float(), _oracle(wl, slopes).float(), atol=ATOL, rtol=RTOL)
@@ -677,3 +738,92 @@ def test_understated_max_sequence_length_cuts_the_context_off(cuda, num_q_heads,
             cut = type(wl)(**{**wl.__dict__, "context_lens": _ctx(512, 100, 512)})
             ref_cut = _oracle(cut, seq_ids=[0])
             torch.testing.assert_close(out[0].float().cpu(), ref_cut[0].float(), atol=ATOL, rtol=RTOL)
+
+
+def _set_token_scales(wl, which, fn):
+    """Replaces the per-token K or V scale of token tau of every sequence by fn(tau) (a tensor of ctx values)."""
+    sc = getattr(wl, which).clone()
+    for b in range(wl.batch):
+        ctx = int(wl.context_lens[b])
+        tau = torch.arange(ctx)
+        pages = wl.block_tables[b, tau // wl.block_size].long()
+        sc[pages, :, tau % wl.block_size, 0] = fn(tau)[:, None].expand(ctx, sc.shape[1])
+    return type(wl)(**{**wl.__dict__, which: sc})
+
+
+def _adversarial(wl, kind):
+    """Data built to drive the softmax bookkeeping of the kernels to its corners; returns (workload, alibi slopes)."""
+    step = lambda tau: tau // 64  # the kernels work in steps of 64 tokens
+    slopes = None
+    if kind in ("gain64", "gain64_vscales"):
+        # logits of +-200: step maxima jump up and down by tens of powers of two, the softmax is nearly one-hot
+        wl = type(wl)(**{**wl.__dict__, "query": (wl.query.float() * 64.0).to(wl.query.dtype)})
+    if kind == "alibi2":
+        # the bias climbs 128 (184 powers of two) per 64-token step: every step lies > 60 powers of two above the last
+        slopes = torch.full((wl.query.shape[1],), 2.0)
+    if kind == "kscale_waves":
+        # per-token K scales x1, x64, x1, ... by step under a query gain of 8: step maxima rise by more than 60
+        # powers of two from one step to the next and fall by as much in the one after
+        wl = type(wl)(**{**wl.__dict__, "query": (wl.query.float() * 8.0).to(wl.query.dtype)})
+        base = wl.key_scale
+        wl = _set_token_scales(wl, "key_scale", lambda tau: float(base.mean()) * torch.where(step(tau) % 2 == 1, 64.0, 1.0))
+    if kind in ("vscales", "gain64_vscales"):
+        # per-token V scales 2^-40 ... 2^+40 ... 2^-40 inside one partition: a triangle over the steps, and +-3 powers of
+        # two from token to token
+        def vs(tau):
+            ns = int(step(tau).max()) + 1
+            tri = 40.0 - 80.0 * (step(tau).float() / max(ns - 1, 1) - 0.5).abs() * 2.0 if ns > 1 else torch.zeros(len(tau))
+            return torch.exp2(torch.round(tri) + (tau % 7).float() - 3.0)
+        wl = _set_token_scales(wl, "value_scale", vs)
+    if kind == "vscales_rising":
+        # V scales that only grow, 2^-60 to 2^+60: the accumulator's unit has to follow them up
+        wl = _set_token_scales(wl, "value_scale", lambda tau: torch.exp2(torch.round(-60.0 + 120.0 * tau.float() / max(len(tau) - 1, 1))))
+    if kind == "vscales_falling_logits_rising":
+        # the V scales fall by 2^100 while the logits climb by as much: each alone is far outside the window the
+        # kernel follows without re-basing, together they cancel and every token carries about the same weight
+        wl = type(wl)(**{**wl.__dict__, "query": (wl.query.float() * 0.0).to(wl.query.dtype)})
+        n_tok = lambda tau: max(len(tau) - 1, 1)
+        wl = _set_token_scales(wl, "value_scale", lambda tau: torch.exp2(50.0 - torch.round(100.0 * tau.float() / n_tok(tau))))
+        slopes = torch.full((wl.query.shape[1],), 100.0 * math.log(2.0) / max(int(wl.context_lens.max()) - 1, 1))
+    return wl, slopes
+
+
+@pytest.mark.parametrize("rows", ["g8_q1", "g8_q4", "g16_q4", "g16_q3_bs1024"])
+@pytest.mark.parametrize("kind", ["gain64", "alibi2", "kscale_waves", "vscales", "gain64_vscales", "vscales_rising",
+                                  "vscales_falling_logits_rising"])
+def test_adversarial_softmax_levels(cuda, kind, rows):
+    """The softmax state of the kernels under data that drives it to its corners: logits that jump by more than 60
+    powers of two between 64-token steps, up and down; per-token V scales that span 2^-40 ... 2^+40 (and 2^-60 ...
+    2^+60) inside one partition; both at once; V scales and logits that drift 100 powers of two in opposite
+    directions.  8 query rows per kv head run pa_partition_kernel (running maximum), 32 rows the shared-stream
+    kernel with two waves per row tile, 64 and 48 rows with one (reference maximum that is re-based).  Every output
+    must be finite and meet the oracle at the usual bar, measured against each row's own magnitude (the outputs
+    reach 2^40); the partition buffers are held against the oracle's partition stage."""
+    g, q_len, bs = dict(g8_q1=(8, 1, 16), g8_q4=(8, 4, 16), g16_q4=(16, 4, 16), g16_q3_bs1024=(16, 3, 1024))[rows]
+    wl = _make(batch=3, num_q_heads=2 * g, num_kv_heads=2, context_lens=_ctx(2048, 700, 1030), q_len=q_len,
+               scale_mode="token", block_size=bs, seed=17)
+    wl, slopes = _adversarial(wl, kind)
+    ref = _oracle(wl, slopes).float()
+    assert bool(torch.isfinite(ref).all())
+    mag = ref.abs().amax(dim=-1, keepdim=True).clamp_min(1e-30)
+    for ps in (2048, 512):
+        print(f"kind={kind} rows={rows} partition_size={ps}", flush=True)
+        out, res = _run(wl, cuda, partition_size=ps, alibi=slopes)
+        o = out.float()
+        assert bool(torch.isfinite(o).all()), "non-finite output"
+        torch.testing.assert_close(o / mag, ref / mag, atol=ATOL, rtol=RTOL)
+        P = res["maximum_logits"].shape[2]
+        ml, es, to = O.partition_stage(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                       wl.softmax_scale, wl.q_len, wl.key_scale, wl.value_scale, slopes, ps, P, q_max=wl.q_len)
+        gml, ges, gto = res["maximum_logits"].cpu(), res["exponential_sums"].cpu(), res["temporary_output"].float().cpu()
+        reach = (torch.arange(P)[None, :] * ps < wl.context_lens[:, None])[:, None, :, None].expand_as(ml)
+        fin = torch.isfinite(ml) & reach
+        assert torch.equal(gml[reach & ~torch.isfinite(ml)], ml[reach & ~torch.isfinite(ml)])
+        # (logits in the hundreds carry f32 rounding of a few 1e-3 absolute, in the kernel and in the oracle alike, and
+        # a near one-hot softmax turns that into parts in a hundred of the sum of exponentials)
+        torch.testing.assert_close(gml[fin], ml[fin], atol=2e-3, rtol=2e-4)
+        torch.testing.assert_close(ges[reach], es[reach], atol=2e-3, rtol=2e-2)
+        tmag = to.abs().amax(dim=-1, keepdim=True).clamp_min(1e-30)
+        assert bool(torch.isfinite(gto[reach[..., None].expand_as(to)]).all())
+        sel = reach[..., None].expand_as(to)
+        torch.testing.assert_close((gto / tmag)[sel], (to / tmag)[sel], atol=ATOL, rtol=RTOL)

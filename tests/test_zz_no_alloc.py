@@ -1,13 +1,15 @@
 """pa_decode_noalloc, the entry point that allocates nothing: its output must equal pa_decode's bit for bit (the
-same kernels run on the same inputs; only where the partition buffers live differs), on two calls in a row that
-share the library's scratch array, the second with a smaller input, and a call too large for the array must be
-refused before anything is launched."""
+same kernels run on the same inputs; only where the partition buffers live differs) and the CPU oracle's within
+the parity bar, on two calls in a row that share the library's scratch array, the second with a smaller input;
+the device's free memory must not move across a call; a call captured into a HIP graph must replay to the same
+bits; and a call too large for the array must be refused before anything is launched."""
 import ctypes as C
 
 import pytest
 import torch
 
 import triton_op_amd as T
+from oracle import pa_oracle as O
 from triton_op_amd import _cabi
 from triton_op_amd import workloads as W
 
@@ -47,13 +49,54 @@ def test_noalloc_matches_pa_decode_on_two_calls_in_a_row():
         # poison this plan's own buffers: the entry point must not touch them
         plan.tmp_output.fill_(float("nan"))
         plan.exp_sums.fill_(float("nan"))
-        before = torch.cuda.memory_allocated(dev)
-        plan.run_noalloc(stream.cuda_stream)
-        assert torch.cuda.memory_allocated(dev) == before
+        plan.run_noalloc(stream.cuda_stream)  # the first call on a device looks the scratch array's address up
         torch.cuda.synchronize()
+        out.fill_(float("nan"))
+        # free device memory as the driver reports it (torch's own counters only see torch's allocator): a
+        # hipMalloc inside the library would move it
+        free_before, _ = torch.cuda.mem_get_info(dev)
+        torch_before = torch.cuda.memory_allocated(dev)
+        plan.run_noalloc(stream.cuda_stream)
+        torch.cuda.synchronize()
+        free_after, _ = torch.cuda.mem_get_info(dev)
+        assert free_after == free_before, (free_before, free_after)
+        assert torch.cuda.memory_allocated(dev) == torch_before
         assert not torch.isnan(out.float()).any()
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), wl.name
         assert torch.isnan(plan.tmp_output.float()).all() and torch.isnan(plan.exp_sums).all()
+        # ... and against the CPU oracle, like every other entry point
+        c = wl.to("cpu")
+        oracle = O.paged_attention_decode_oracle(c.query, c.key_cache, c.value_cache, c.context_lens, c.block_tables,
+                                                 c.softmax_scale, c.q_len if c.q_lens is None else c.q_lens, c.key_scale,
+                                                 c.value_scale, q_max=c.q_len)
+        torch.testing.assert_close(out.float().cpu(), oracle.float(), atol=2e-2, rtol=2e-2)
+
+
+def test_noalloc_call_captured_in_a_graph_replays_to_the_same_bits():
+    """The entry point is for callers under graph capture.  One call is made outside capture first (the first call
+    on a device asks the runtime for the scratch array's address); then a call is captured and replayed three
+    times with eager work and host synchronisations in between, each replay held against pa_decode's result."""
+    dev = torch.device("cuda:0")
+    (wl, ps), _ = _workloads(dev)
+    ref = torch.full_like(wl.query, float("nan"))
+    _plan(wl, ref, ps).run()
+    out = torch.full_like(wl.query, float("nan"))
+    plan = _plan(wl, out, ps)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        plan.run_noalloc(side.cuda_stream)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            plan.run_noalloc(side.cuda_stream)
+    torch.cuda.synchronize()
+    for i in range(3):
+        out.fill_(float("nan"))
+        (wl.key_cache.float()[:1] * 1.0).sum().item()  # unrelated eager work and a host sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"replay {i}"
 
 
 def test_noalloc_refuses_what_does_not_fit():

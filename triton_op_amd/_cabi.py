@@ -12,7 +12,7 @@ import threading
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
-PA_DECODE_ABI_VERSION = 4
+PA_DECODE_ABI_VERSION = 5
 PA_DECODE_WORKSPACE_BYTES = 64
 PA_DECODE_NOALLOC_SCRATCH_BYTES = 64 << 20
 PA_ERR_SCRATCH_TOO_SMALL = -7
@@ -33,8 +33,6 @@ EXPORTED_SYMBOLS = (
     "pa_decode_noalloc",
     "pa_decode_launch_info",
     "pa_debug_fp8_decode",
-    "pa_debug_gather_probe",
-    "pa_debug_issue_probe",
     "pa_kv_cache_write",
     "pa_quantize_kv_cache",
 )
@@ -50,7 +48,7 @@ class PaDecodeArgs(C.Structure):
         + [(n, C.c_int32) for n in (
             "num_seqs", "num_kv_heads", "group_size", "q_len", "head_size", "block_size",
             "max_num_partitions", "partition_size", "query_dtype", "kv_dtype", "query_quant_mode",
-            "kv_quant_mode", "v_transposed")]
+            "kv_quant_mode", "v_transposed", "alibi_slopes_len", "reserved0")]
         + [("softmax_scale", C.c_float)]
         + [(n, C.c_int64) for n in (
             "stride_out_s", "stride_out_h", "stride_q_s", "stride_q_h",
@@ -109,10 +107,6 @@ def load_library(path: str = None) -> C.CDLL:
             fn.argtypes = [C.POINTER(PaDecodeArgs), C.c_void_p]
         lib.pa_decode_launch_info.restype = C.c_int
         lib.pa_decode_launch_info.argtypes = [C.POINTER(PaDecodeArgs), C.c_char_p, C.c_int32]
-        lib.pa_debug_gather_probe.restype = C.c_int
-        lib.pa_debug_gather_probe.argtypes = [C.POINTER(PaDecodeArgs), C.c_void_p, C.c_void_p]
-        lib.pa_debug_issue_probe.restype = C.c_int
-        lib.pa_debug_issue_probe.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
         lib.pa_debug_fp8_decode.restype = C.c_int
         lib.pa_debug_fp8_decode.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
         lib.pa_kv_cache_write.restype = C.c_int

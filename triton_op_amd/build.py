@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = [os.path.join(HERE, "csrc", "pa_decode.hip"), os.path.join(HERE, "csrc", "pa_kv_cache.hip")]
 HEADERS = [os.path.join(HERE, "..", "include", "pa_decode.h")] + [
     os.path.join(HERE, "csrc", h)
-    for h in ("pa_common.h", "pa_partition_kernel.h", "pa_partition_shared_kernel.h", "pa_plan_kernel.h", "pa_probe_kernel.h",
+    for h in ("pa_common.h", "pa_launch.h", "pa_partition_kernel.h", "pa_partition_shared_kernel.h", "pa_plan_kernel.h",
               "pa_reduce_kernel.h")]
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
@@ -69,6 +69,22 @@ def build_native_smoke(verbose: bool = True) -> str:
     return NATIVE_SMOKE_BIN
 
 
+PROBE_SRC = os.path.join(HERE, "..", "tests", "native", "pa_probe.hip")
+PROBE_LIB = os.path.join(HERE, "..", "tests", "native", "libpa_probe.so")
+
+
+def build_probe(verbose: bool = True) -> str:
+    """The measuring kernels of bench.py's probe workloads (tests/native/pa_probe.h): a library of their own, built
+    from the decode kernels' headers; not part of the operator or its ABI."""
+    cmd = [find_hipcc(), *HIPCC_FLAGS, PROBE_SRC, "-o", PROBE_LIB]
+    if verbose:
+        print("[triton_op_amd.build]", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
+    return PROBE_LIB
+
+
 def is_stale() -> bool:
     if not os.path.exists(LIB_PATH):
         return True
@@ -79,3 +95,4 @@ def is_stale() -> bool:
 if __name__ == "__main__":
     build()
     build_native_smoke()
+    build_probe()

@@ -17,16 +17,18 @@
 
 #include "../../include/pa_decode.h"
 #include "pa_common.h"
+#include "pa_launch.h"
 #include "pa_partition_kernel.h"
 #include "pa_partition_shared_kernel.h"
 #include "pa_plan_kernel.h"
-#include "pa_probe_kernel.h"
 #include "pa_reduce_kernel.h"
 
 // Scratch of pa_decode_noalloc, the entry point for callers that can neither allocate nor pass partition buffers:
 // the item-list workspace and the three partition buffers of one call.  Every GPU the library runs on holds its
 // own copy at its own address; host code reaches it only through the address hipGetSymbolAddress returns there.
 static __device__ __align__(256) unsigned char scratch[PA_DECODE_NOALLOC_SCRATCH_BYTES];
+
+thread_local int pa_last_hip_error = 0;
 
 namespace {
 
@@ -47,8 +49,6 @@ __global__ void pa_fp8_decode_kernel(const uint8_t* codes, float* out, int n) {
   float b = bf16_bits_to_f32(hi & 0xffffu);
   out[i] = (i & 1) ? b : a;
 }
-
-thread_local int g_last_hip_error = 0;
 
 int check_common(const PaDecodeArgs* a) {
   if (!a) return PA_ERR_NULL_POINTER;
@@ -228,46 +228,35 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
   return c;
 }
 
-int launch_status() {
-  const hipError_t e = hipGetLastError();
-  if (e == hipSuccess) return PA_OK;
-  g_last_hip_error = (int)e;
-  return PA_ERR_LAUNCH;
-}
-
 int launch_plan(const PaDecodeArgs& a, hipStream_t stream) {
-  hipLaunchKernelGGL(pa_plan_kernel, dim3(1), dim3(1024), 0, stream, a);
-  return launch_status();
+  return pa_launch(pa_plan_kernel, dim3(1), dim3(1024), 0, stream, a);
 }
 
 // pa_partition_kernel is instantiated with one 16-row query tile per workgroup (NT = 1): a bf16 cache with
 // more than 16 query rows per kv head gets one workgroup per tile (they read the same pages at the same time
 // from the same L2, and tiles that hold only padding rows cost nothing).
 template <int NT, int KVT, bool PT, bool BS16, int W>
-void launch_partition_w(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+int launch_partition_w(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
   constexpr int OCC = NT == 1 ? 2 : 1;
   if (c.queue)
-    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
-                       stream, k);
-  else
-    hipLaunchKernelGGL((pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>), dim3((unsigned)c.blocks), dim3(64 * W), 0,
-                       stream, k);
+    return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>, dim3((unsigned)c.blocks), dim3(64 * W), 0, stream, k);
+  return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>, dim3((unsigned)c.blocks), dim3(64 * W), 0, stream, k);
 }
 
 template <int NT, int KVT, bool PT, bool BS16>
-void launch_partition_tile(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+int launch_partition_tile(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
   if (c.waves == 4) return launch_partition_w<NT, KVT, PT, BS16, 4>(k, c, stream);
   if (c.waves == 2) return launch_partition_w<NT, KVT, PT, BS16, 2>(k, c, stream);
   return launch_partition_w<NT, KVT, PT, BS16, 1>(k, c, stream);
 }
 
 template <bool PT, bool BS16>
-void launch_partition_shared(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+int launch_partition_shared(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
   static const int pad = debug_switch("PA_DECODE_LDS_PAD", 0);  // experiment: unused LDS that lowers the occupancy
   if constexpr (PT)
-    hipLaunchKernelGGL((pa_partition_shared_kernel<true, BS16, 3, 3>), dim3((unsigned)c.blocks), dim3(256), pad, stream, k);
+    return pa_launch(pa_partition_shared_kernel<true, BS16, 3, 3>, dim3((unsigned)c.blocks), dim3(256), (unsigned)pad, stream, k);
   else
-    hipLaunchKernelGGL((pa_partition_shared_kernel<false, BS16, 2, 4>), dim3((unsigned)c.blocks), dim3(256), pad, stream, k);
+    return pa_launch(pa_partition_shared_kernel<false, BS16, 2, 4>, dim3((unsigned)c.blocks), dim3(256), (unsigned)pad, stream, k);
 }
 
 // stage 1 as chosen: the planning kernel when the items are to be sorted, then the partition kernel
@@ -287,23 +276,19 @@ int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t s
   }
   if (c.span > 1) k.flags |= c.span << kFlagSpanShift;
   if (!c.fp8) {
-    if (c.row_tiles == 2)
-      launch_partition_tile<2, PA_DTYPE_BF16, false, false>(k, c, stream);
-    else
-      launch_partition_tile<1, PA_DTYPE_BF16, false, false>(k, c, stream);
-  } else if (c.shared) {
-    if (c.bs16)
-      c.per_token ? launch_partition_shared<true, true>(k, c, stream) : launch_partition_shared<false, true>(k, c, stream);
-    else
-      c.per_token ? launch_partition_shared<true, false>(k, c, stream) : launch_partition_shared<false, false>(k, c, stream);
-  } else if (c.bs16) {
-    c.per_token ? launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, true, true>(k, c, stream)
-                : launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, false, true>(k, c, stream);
-  } else {
-    c.per_token ? launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, true, false>(k, c, stream)
-                : launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, false, false>(k, c, stream);
+    if (c.row_tiles == 2) return launch_partition_tile<2, PA_DTYPE_BF16, false, false>(k, c, stream);
+    return launch_partition_tile<1, PA_DTYPE_BF16, false, false>(k, c, stream);
   }
-  return launch_status();
+  if (c.shared) {
+    if (c.bs16)
+      return c.per_token ? launch_partition_shared<true, true>(k, c, stream) : launch_partition_shared<false, true>(k, c, stream);
+    return c.per_token ? launch_partition_shared<true, false>(k, c, stream) : launch_partition_shared<false, false>(k, c, stream);
+  }
+  if (c.bs16)
+    return c.per_token ? launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, true, true>(k, c, stream)
+                       : launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, false, true>(k, c, stream);
+  return c.per_token ? launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, true, false>(k, c, stream)
+                     : launch_partition_tile<1, PA_DTYPE_FP8_E4M3FN, false, false>(k, c, stream);
 }
 
 // the argument checks of stage 1
@@ -320,6 +305,10 @@ int check_partition(const PaDecodeArgs* a) {
     return PA_ERR_UNSUPPORTED;
   if (a->kv_quant_mode == PA_QUANT_PER_TOKEN && a->kv_dtype != PA_DTYPE_FP8_E4M3FN)
     return PA_ERR_UNSUPPORTED;  // per-token scales belong to the FP8 cache
+  // ALiBi: one slope per packed query row (the reference kernels' array) or one per query head
+  if (a->alibi_slopes && a->alibi_slopes_len != a->num_kv_heads * a->q_len * a->group_size &&
+      a->alibi_slopes_len != a->num_kv_heads * a->group_size)
+    return PA_ERR_BAD_SHAPE;
   const int esz = a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? 1 : 2;
   // 16-byte vector loads: every stride that moves a vector must keep it 16-byte aligned
   if ((a->stride_k_b * esz) % 16 || (a->stride_k_h * esz) % 16 || (a->stride_k_c * esz) % 16 ||
@@ -358,23 +347,12 @@ int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
   // enough rows to fill the GPU's wave slots several times over: four rows per wave
   const bool big = blocks * 16 >= 16384;
-  if (skip_single) {
-    if (big)
-      hipLaunchKernelGGL((pa_reduce_kernel<true, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, *a);
-    else
-      hipLaunchKernelGGL((pa_reduce_kernel<true, 1>), dim3((unsigned)blocks), dim3(1024), 0, stream, *a);
-  } else {
-    if (big)
-      hipLaunchKernelGGL((pa_reduce_kernel<false, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, *a);
-    else
-      hipLaunchKernelGGL((pa_reduce_kernel<false, 1>), dim3((unsigned)blocks), dim3(1024), 0, stream, *a);
-  }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
+  const dim3 grid((unsigned)blocks);
+  if (skip_single)
+    return big ? pa_launch(pa_reduce_kernel<true, 4>, grid, dim3(256), 0, stream, *a)
+               : pa_launch(pa_reduce_kernel<true, 1>, grid, dim3(1024), 0, stream, *a);
+  return big ? pa_launch(pa_reduce_kernel<false, 4>, grid, dim3(256), 0, stream, *a)
+             : pa_launch(pa_reduce_kernel<false, 1>, grid, dim3(1024), 0, stream, *a);
 }
 
 // The reduce stage of a call whose partition stage went through the planning kernel: only the sequences with
@@ -384,16 +362,8 @@ int launch_reduce_listed(const PaDecodeArgs* a, void* hip_stream) {
   const long long cap = 8LL * device_num_cus();
   const unsigned blocks = (unsigned)(units < cap ? units : cap);
   hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-  if (units * 16 >= 16384)
-    hipLaunchKernelGGL((pa_reduce_listed_kernel<4>), dim3(blocks), dim3(256), 0, stream, *a);
-  else
-    hipLaunchKernelGGL((pa_reduce_listed_kernel<1>), dim3(blocks), dim3(1024), 0, stream, *a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
+  if (units * 16 >= 16384) return pa_launch(pa_reduce_listed_kernel<4>, dim3(blocks), dim3(256), 0, stream, *a);
+  return pa_launch(pa_reduce_listed_kernel<1>, dim3(blocks), dim3(1024), 0, stream, *a);
 }
 
 }  // namespace
@@ -402,7 +372,7 @@ extern "C" {
 
 int pa_decode_abi_version(void) { return PA_DECODE_ABI_VERSION; }
 uint32_t pa_decode_args_size(void) { return (uint32_t)sizeof(PaDecodeArgs); }
-int pa_decode_last_hip_error(void) { return g_last_hip_error; }
+int pa_decode_last_hip_error(void) { return pa_last_hip_error; }
 
 int64_t pa_decode_workspace_bytes(int32_t num_seqs, int32_t max_num_partitions) {
   if (num_seqs <= 0 || max_num_partitions <= 0) return PA_DECODE_WORKSPACE_BYTES;
@@ -540,16 +510,33 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
   if (a->struct_size != sizeof(PaDecodeArgs)) return PA_ERR_BAD_STRUCT;
   // the library owns these four in this entry point: a caller that passes its own wants pa_decode
   if (a->exp_sums || a->max_logits || a->tmp_output || a->workspace || a->workspace_bytes) return PA_ERR_BAD_SHAPE;
-  if (a->num_seqs <= 0 || a->num_kv_heads <= 0 || a->group_size <= 0 || a->q_len <= 0 || a->max_num_partitions <= 0 ||
-      a->head_size != kHeadSize)
-    return PA_ERR_BAD_SHAPE;
+  // Every other check of pa_decode runs on the caller's arguments first, with stand-ins for the four buffers the
+  // library brings: the sizes below are then products of checked, positive int32 values.
+  {
+    PaDecodeArgs probe = *a;
+    probe.exp_sums = probe.max_logits = reinterpret_cast<float*>(uintptr_t{256});
+    probe.tmp_output = reinterpret_cast<void*>(uintptr_t{256});
+    probe.stride_es_s = probe.stride_es_h = probe.stride_es_p = 0;  // the caller's strides of these buffers are ignored
+    probe.stride_tmp_s = probe.stride_tmp_h = probe.stride_tmp_p = probe.stride_tmp_g = 0;
+    int rc = check_partition(&probe);
+    if (rc) return rc;
+    rc = check_reduce(&probe);
+    if (rc) return rc;
+  }
 
-  // ---- this device's copy of the scratch array: its address is asked for once per device, with that device current
+  // ---- this device's copy of the scratch array: its address is asked for once per device, with that device
+  // current.  The stream must belong to the current device (a stream of another GPU would get a pointer into the
+  // wrong GPU's array): checked, not assumed.
   constexpr int kMaxDevices = 64;
   static unsigned char* scratch_of_device[kMaxDevices] = {};
   static std::mutex scratch_lock;
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return PA_ERR_NO_DEVICE;
+  if (hip_stream != nullptr) {
+    int stream_dev = -1;
+    if (hipStreamGetDevice(reinterpret_cast<hipStream_t>(hip_stream), &stream_dev) != hipSuccess || stream_dev != dev)
+      return PA_ERR_NO_DEVICE;
+  }
   unsigned char* base;
   {
     std::lock_guard<std::mutex> guard(scratch_lock);
@@ -557,7 +544,7 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
       void* p = nullptr;
       const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
       if (e != hipSuccess || !p) {
-        g_last_hip_error = (int)e;
+        pa_last_hip_error = (int)e;
         return PA_ERR_LAUNCH;
       }
       scratch_of_device[dev] = static_cast<unsigned char*>(p);
@@ -566,15 +553,22 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
   }
 
   // ---- layout: workspace, max_logits, exp_sums, tmp_output, each at a multiple of 256 bytes ------------------
+  // (the four factors are positive int32 values and ge <= 64: every product is formed with an overflow check)
   const auto round256 = [](long long n) { return (n + 255) / 256 * 256; };
   const long long ge = (long long)a->q_len * a->group_size;
-  const long long rows = (long long)a->num_seqs * a->num_kv_heads * a->max_num_partitions * ge;
+  const long long limit = (long long)PA_DECODE_NOALLOC_SCRATCH_BYTES;
+  long long rows = 0, tmp_bytes = 0;
+  if (__builtin_mul_overflow((long long)a->num_seqs * a->num_kv_heads, (long long)a->max_num_partitions * ge, &rows) ||
+      __builtin_mul_overflow(rows, 2LL * kHeadSize, &tmp_bytes) || tmp_bytes > limit)
+    return PA_ERR_SCRATCH_TOO_SMALL;
+  // (rows * 256 <= 64 MiB bounds num_seqs * max_num_partitions by 2^18: the workspace size cannot overflow either)
   const long long ws_bytes = full_workspace_bytes(a->num_seqs, a->max_num_partitions);
+  if (ws_bytes > limit) return PA_ERR_SCRATCH_TOO_SMALL;
   const long long off_ml = round256(ws_bytes);
   const long long off_es = off_ml + round256(4 * rows);
   const long long off_tmp = off_es + round256(4 * rows);
-  const long long total = off_tmp + round256(2 * rows * kHeadSize);
-  if (total > (long long)PA_DECODE_NOALLOC_SCRATCH_BYTES) return PA_ERR_SCRATCH_TOO_SMALL;
+  const long long total = off_tmp + round256(tmp_bytes);
+  if (total > limit) return PA_ERR_SCRATCH_TOO_SMALL;
 
   PaDecodeArgs k = *a;
   k.workspace = reinterpret_cast<int32_t*>(base);
@@ -592,58 +586,17 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
   // the array keeps the last call's contents (a call that was cut short may have left its counters non-zero, and
   // an item list of another batch): the counters are cleared, the lists are rebuilt
   k.flags &= ~PA_DECODE_FLAG_REUSE_ITEM_LIST;
-  hipLaunchKernelGGL(pa_clear_words_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(hip_stream),
-                     k.workspace, kPlanHeaderWords);
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return pa_decode(&k, hip_stream);
-}
-
-int pa_debug_gather_probe(const PaDecodeArgs* a, int32_t* sink, void* hip_stream) {
-  const int rc = check_partition(a);
+  const int rc = pa_launch(pa_clear_words_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(hip_stream),
+                           k.workspace, (int)kPlanHeaderWords);
   if (rc) return rc;
-  if (!sink) return PA_ERR_NULL_POINTER;
-  if (a->kv_dtype != PA_DTYPE_FP8_E4M3FN || a->block_size != 16 || a->stride_k_c != 256 || a->stride_v_2 != 16 ||
-      a->v_transposed)
-    return PA_ERR_UNSUPPORTED;
-  const long long blocks = (long long)a->num_seqs * a->num_kv_heads * a->max_num_partitions;
-  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(pa_gather_probe_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                     reinterpret_cast<hipStream_t>(hip_stream), *a, sink);
-  return launch_status();
-}
-
-int pa_debug_issue_probe(int32_t mode, int32_t iterations, int32_t workgroups, int32_t* sink, void* hip_stream) {
-  if (!sink) return PA_ERR_NULL_POINTER;
-  if (iterations <= 0 || workgroups <= 0) return PA_ERR_BAD_SHAPE;
-  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-  const dim3 grid((unsigned)workgroups), block(256);
-  switch (mode) {
-    case 0: hipLaunchKernelGGL(pa_issue_probe_kernel<0>, grid, block, 0, stream, sink, iterations); break;
-    case 1: hipLaunchKernelGGL(pa_issue_probe_kernel<1>, grid, block, 0, stream, sink, iterations); break;
-    case 2: hipLaunchKernelGGL(pa_issue_probe_kernel<2>, grid, block, 0, stream, sink, iterations); break;
-    case 3: hipLaunchKernelGGL(pa_issue_probe_kernel<3>, grid, block, 0, stream, sink, iterations); break;
-    case 4: hipLaunchKernelGGL(pa_issue_probe_kernel<4>, grid, block, 0, stream, sink, iterations); break;
-    case 5: hipLaunchKernelGGL(pa_issue_probe_kernel<5>, grid, block, 0, stream, sink, iterations); break;
-    default: return PA_ERR_UNSUPPORTED;
-  }
-  return launch_status();
+  return pa_decode(&k, hip_stream);
 }
 
 int pa_debug_fp8_decode(const uint8_t* codes, float* out, int32_t n, void* hip_stream) {
   if (!codes || !out) return PA_ERR_NULL_POINTER;
   if (n <= 0) return PA_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(pa_fp8_decode_kernel, dim3((n + 255) / 256), dim3(256), 0,
-                     reinterpret_cast<hipStream_t>(hip_stream), codes, out, n);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
+  return pa_launch(pa_fp8_decode_kernel, dim3((n + 255) / 256), dim3(256), 0, reinterpret_cast<hipStream_t>(hip_stream),
+                   codes, out, (int)n);
 }
 
 }  // extern "C"

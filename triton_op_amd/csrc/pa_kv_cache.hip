@@ -10,6 +10,7 @@
 #include <stdint.h>
 
 #include "../../include/pa_decode.h"
+#include "pa_launch.h"
 
 namespace {
 
@@ -475,8 +476,6 @@ __global__ __launch_bounds__(256) void quantize_kv_cache_kernel(const uint16_t* 
     vo[(int64_t)d * bs + tok] = f32_to_fp8(__fdiv_rn(bf16_to_f32(vp[(int64_t)d * bs + tok]), vs));
 }
 
-thread_local int g_last_hip_error_kv = 0;
-
 }  // namespace
 
 extern "C" {
@@ -516,23 +515,14 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
     const long long head_groups = (a->num_kv_heads + hpw - 1) / hpw;
     if (windows * head_groups > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
     const dim3 grid((unsigned)(windows * head_groups));
-    if (per_token)
-      hipLaunchKernelGGL((kv_cache_write_tile_kernel<true, 2>), grid, dim3(256), 0, stream, *a, regroup, bs_shift);
-    else if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
-      hipLaunchKernelGGL((kv_cache_write_tile_kernel<true, 4>), grid, dim3(256), 0, stream, *a, regroup, bs_shift);
-    else
-      hipLaunchKernelGGL((kv_cache_write_tile_kernel<false, 4>), grid, dim3(256), 0, stream, *a, regroup, bs_shift);
-  } else if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN) {
-    hipLaunchKernelGGL(kv_cache_write_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
-  } else {
-    hipLaunchKernelGGL(kv_cache_write_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
+    if (per_token) return pa_launch(kv_cache_write_tile_kernel<true, 2>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
+    if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
+      return pa_launch(kv_cache_write_tile_kernel<true, 4>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
+    return pa_launch(kv_cache_write_tile_kernel<false, 4>, grid, dim3(256), 0, stream, *a, regroup, bs_shift);
   }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error_kv = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
+  if (a->cache_dtype == PA_DTYPE_FP8_E4M3FN)
+    return pa_launch(kv_cache_write_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
+  return pa_launch(kv_cache_write_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, *a);
 }
 
 int pa_quantize_kv_cache(const void* key_cache_bf16, const void* value_cache_bf16, void* key_cache_fp8,
@@ -568,20 +558,13 @@ int pa_quantize_kv_cache(const void* key_cache_bf16, const void* value_cache_bf1
     const int regroup = block_size > 16;
     const long long grid = regroup ? (num_windows + 63) / 64 * 64 : num_windows;
     if (grid > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-    hipLaunchKernelGGL(quantize_kv_cache_tile_kernel, dim3((unsigned)grid), dim3(256), 0, stream, a, num_windows, regroup);
-  } else {
-    const long long blocks = (n + 255) / 256;
-    if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-    hipLaunchKernelGGL(quantize_kv_cache_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                       (const uint16_t*)key_cache_bf16, (const uint16_t*)value_cache_bf16, (uint8_t*)key_cache_fp8,
-                       (uint8_t*)value_cache_fp8, key_scale, value_scale, (long long)num_blocks * num_kv_heads, block_size);
+    return pa_launch(quantize_kv_cache_tile_kernel, dim3((unsigned)grid), dim3(256), 0, stream, a, num_windows, regroup);
   }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    g_last_hip_error_kv = (int)e;
-    return PA_ERR_LAUNCH;
-  }
-  return PA_OK;
+  const long long blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  return pa_launch(quantize_kv_cache_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)key_cache_bf16,
+                   (const uint16_t*)value_cache_bf16, (uint8_t*)key_cache_fp8, (uint8_t*)value_cache_fp8, key_scale,
+                   value_scale, (long long)num_blocks * num_kv_heads, (int)block_size);
 }
 
 }  // extern "C"

@@ -333,13 +333,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   int limit[NT];      // number of visible keys of this lane's query row
   float slope2[NT];   // ALiBi slope * log2e
   const bool has_alibi = a.alibi_slopes != nullptr;
+  const bool alibi_per_row = a.alibi_slopes_len == Hkv * Ge;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     int row = row0 + 16 * nt + li;
     int t = row / G;
     limit[nt] = row < rows_valid ? ctx - (qb - 1 - t) : 0;
     slope2[nt] = 0.f;
-    if (has_alibi && row < rows_valid) slope2[nt] = a.alibi_slopes[h * G + (row - t * G)] * kLog2e;
+    // one slope per packed row (the reference kernels' indexing) or one per query head, shared by its new tokens
+    if (has_alibi && row < rows_valid)
+      slope2[nt] = a.alibi_slopes[alibi_per_row ? h * Ge + row : h * G + (row - t * G)] * kLog2e;
   }
   const int min_limit = ctx - (qb - 1);  // keys below this index are visible to every real row
 
@@ -441,14 +444,22 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       }
     }
   }
-  float v_run;          // FP8 math with per-token V scales: running max of the scales seen so far
+  // FP8 math with per-token V scales: the unit the row's accumulator is kept in.  A step's P * v_scale is at most
+  // (the step's largest P) * (the step's largest scale); the unit is that bound, unless the accumulator, decayed
+  // by alpha like everything the row has seen, still needs a larger one:
+  //     v_run <- max(vmx * exp2(step max - running max), v_run * alpha).
+  // So P * v_scale / v_run never exceeds 1 and the step's own largest term is never far below it, whichever way
+  // logits and scales drift against each other over a partition (a fixed unit, the running maximum of the scales,
+  // loses a late token that carries the result through a large V scale but lies below an early token's logit).
+  // Floored at 1e-30.
+  float v_run[NT];
   float m_run[NT];      // running max of the scaled logits, log2 domain (-inf before the first visible key)
   float l_run[NT];      // this lane's share of the running sum of exp2(s - m)
   f32x4 acc[NT][8];     // O^T: acc[nt][db][r] is head dim 16*db + 4*kg + r of query row 16*nt + li
   auto reset_state = [&]() {
-    v_run = 1e-30f;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
+      v_run[nt] = 1e-30f;
       m_run[nt] = -INFINITY;
       l_run[nt] = 0.f;
 #pragma unroll
@@ -496,14 +507,12 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     if constexpr (PREFETCH) issue_k(sd, pg_next);
     __builtin_amdgcn_sched_barrier(0);
 
-    // FP8 math, per-token V scales: P carries v_scale / v_run (<= 1); the accumulator is kept in units
-    // of the running maximum v_run
+    // FP8 math, per-token V scales: P carries v_scale / v_run (<= 1); the row's accumulator is kept in units of v_run
     // FP8 math: P is produced already multiplied by pmul = 256 / v_run; log2(pmul) rides in the exponent's
     // additive term, so the factor costs nothing per element
-    float vfac = 1.f, log2_pmul = FP8MATH ? 8.f : 0.f, inv_pmul = FP8MATH ? 1.f / 256.f : 1.f;
     f32x4 vs_cur[(PER_TOKEN && FP8MATH) ? 4 : 1];
+    float vmx = 0.f;  // the largest V scale of the step (the same in every lane)
     if constexpr (PER_TOKEN && FP8MATH) {
-      float vmx = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         vs_cur[j] = sd.vs[j];
@@ -517,11 +526,6 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         }
       }
       vmx = quad_row_max(vmx);
-      const float v_new = fmaxf(v_run, vmx);
-      vfac = v_new == v_run ? 1.f : v_run * __builtin_amdgcn_rcpf(v_new);
-      log2_pmul = 8.f - __builtin_amdgcn_logf(v_new);
-      inv_pmul = v_new * (1.f / 256.f);
-      v_run = v_new;
     }
     uint32_t ph[FP8MATH ? NT : 1][4], pl[FP8MATH ? NT : 1][4];  // FP8 math: P head / residual, 4 tokens per dword
 
@@ -551,6 +555,17 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = fast_exp2(m_run[nt] - m_safe);  // exp2(-inf) = 0 on the first visible step
       m_run[nt] = m_new;
+      float alpha_acc = alpha, log2_pmul = FP8MATH ? 8.f : 0.f, inv_pmul = FP8MATH ? 1.f / 256.f : 1.f;
+      if constexpr (PER_TOKEN && FP8MATH) {
+        // the accumulator has just decayed by alpha: its unit may come down by as much, and no further
+        const float v_old = v_run[nt] * alpha;
+        const float v_step = vmx * fast_exp2(mx - m_safe);  // (0 for a row that sees no key of this step)
+        const float v_new = fmaxf(fmaxf(v_step, v_old), 1e-30f);
+        alpha_acc = v_new == v_old ? 1.f : v_old * __builtin_amdgcn_rcpf(v_new);  // <= 1
+        log2_pmul = 8.f - __builtin_amdgcn_logf(v_new);
+        inv_pmul = v_new * (1.f / 256.f);
+        v_run[nt] = v_new;
+      }
       const float e_add = log2_pmul - m_safe;
       const float e_mul = FULL ? rs : 1.f;
       float psum = 0.f;
@@ -599,7 +614,6 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         *reinterpret_cast<u32x2*>(plds + nt * (16 * kPRowBytes) + li * kPRowBytes + (16 * j + 4 * kg) * 2) = pk;
       }
       l_run[nt] = l_run[nt] * alpha + psum * inv_pmul;
-      const float alpha_acc = alpha * vfac;
 #pragma unroll
       for (int db = 0; db < 8; ++db) acc[nt][db] *= alpha_acc;
     }
@@ -699,9 +713,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     if constexpr (kSpanCapable) {
       if (span > 1 && --steps_left_in_part == 0) {
         // (the one-wave epilogue below, up to the staging in LDS, for a partition that is not the workgroup's last)
-        const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
+          const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run[nt] : 1.f) * (1.f / 256.f) : 1.f;
           char* slot = &span_lds[0] + ((part_cur - part) * NT + nt) * kSpanSlotBytes;
           float l_tot = quad_row_sum(l_run[nt]);
           float m_out = m_run[nt];
@@ -770,10 +784,10 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // cuts off longer contexts for any other length.)
   const bool direct = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
-  const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run : 1.f) * (1.f / 256.f) : 1.f;
-  float l_tot[NT];
+  float l_tot[NT], acc_unit[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
+    acc_unit[nt] = FP8MATH ? (PER_TOKEN ? v_run[nt] : 1.f) * (1.f / 256.f) : 1.f;
     l_tot[nt] = quad_row_sum(l_run[nt]);
     if (row0 + 16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
       l_tot[nt] = 0.f;
@@ -784,7 +798,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       const int row = row0 + 16 * nt + li;
-      const float inv = l_tot[nt] > 0.f ? v_tensor_scale * acc_unit / l_tot[nt] : 0.f;
+      const float inv = l_tot[nt] > 0.f ? v_tensor_scale * acc_unit[nt] / l_tot[nt] : 0.f;
       if (row < Ge && kg == 0) {
         a.max_logits[es_off + row] = m_run[nt] * (1.0f / kLog2e);
         a.exp_sums[es_off + row] = l_tot[nt];
@@ -806,7 +820,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         mg_l[wave][16 * nt + li] = l_tot[nt];
       }
 #pragma unroll
-      for (int db = 0; db < 8; ++db) mg_acc[wave][nt][db][lane] = acc[nt][db] * acc_unit;
+      for (int db = 0; db < 8; ++db) mg_acc[wave][nt][db][lane] = acc[nt][db] * acc_unit[nt];
     }
     __syncthreads();
     constexpr int DBW = 8 / WAVES;

@@ -177,7 +177,9 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int t_row = row / G;
   const int limit = row_ok ? ctx - (qb - 1 - t_row) : 0;  // number of visible keys of this lane's query row
   float slope2 = 0.f;
-  if (has_alibi && row_ok) slope2 = a.alibi_slopes[h * G + (row - t_row * G)] * kLog2e;
+  // one slope per packed row (the reference kernels' indexing) or one per query head, shared by its new tokens
+  if (has_alibi && row_ok)
+    slope2 = a.alibi_slopes[a.alibi_slopes_len == Hkv * Ge ? h * Ge + row : h * G + (row - t_row * G)] * kLog2e;
   const int min_limit = ctx - (qb - 1);
 
   // ---- query: q * cq = hi + lo in e4m3, cq a power of two (exact), the B operand of S^T = K Q^T ---------
@@ -254,11 +256,18 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   // The power of two that brings the step's P V back to the reference, 2^(n + k - k_ref), is the E8M0 block scale of
   // the P operand of the scaled MFMA -- exact, and free.  Nothing is rescaled per step: no exp2 of a maximum's
   // movement, no multiplication of the 32 accumulator registers (with an exact running maximum some row of the
-  // sixteen moves on most steps of a long context).  The reference is re-based only when a step's level has run
-  // more than kMaxAhead powers of two ahead of it (f32 headroom), which ordinary data never does.
+  // sixteen moves on most steps of a long context).  The reference is re-based only when a step's level --
+  // logits and V-scale unit TOGETHER, (max - m_ref) + (k - k_ref) -- has run more than kMaxAhead powers of two
+  // ahead of it, which ordinary data never does.  f32 headroom: a step adds at most 2^(kMaxAhead + 1) (level) x
+  // 2^kPBits (P) x 2^9 (an e4m3 value) x 64 tokens = 2^85 to an accumulator register, and a partition has fewer
+  // than 2^25 steps.  Levels far BELOW the reference cost nothing: P is formed against the step's own level down
+  // to kMaxBehind powers of two under the reference (below that its weight against the reference step's own
+  // contribution to l is under 2^-200), and a block scale that would leave E8M0's range is clamped, which only
+  // misstates terms of under 2^-100 of the accumulator's unit.
   // (m_ref, l) stay a consistent pair; the epilogue restates l against the true maximum for the partition buffers.
-  constexpr int kPBits = 8;          // P is produced times 2^kPBits (at most 256; e4m3 reaches 448)
-  constexpr float kMaxAhead = 60.f;  // n and k - k_ref stay below this
+  constexpr int kPBits = 8;            // P is produced times 2^kPBits (at most 256; e4m3 reaches 448)
+  constexpr float kMaxAhead = 60.f;    // (max - m_ref) + (k - k_ref) stays at or below this
+  constexpr float kMaxBehind = 200.f;  // a step's own level is followed this far down
   float m_ref = -INFINITY;
   float m_ref_safe = 0.f;   // m_ref, or 0 while it is -inf
   float m_true = -INFINITY;
@@ -326,11 +335,14 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     mx = quad_row_max(mx);
     if constexpr (FULL) mx *= rscale;
     m_true = fmaxf(m_true, mx);
-    // the rare step: a row sees its first key, or this step's level is too far ahead of the reference
+    // the rare step: a row sees its first key, or this step's level -- its logits' and its V scales' together -- is
+    // too far ahead of the reference.  Then the V-scale unit moves to this step's, and every row whose maximum
+    // lies above its reference moves the reference up to it.
     float ahead = mx - m_ref;  // +inf at a row's first visible key, NaN while it has seen none (compares false)
-    if (__builtin_amdgcn_ballot_w64(ahead > kMaxAhead) != 0 || k - k_ref > (int)kMaxAhead) {
+    const float level = PER_TOKEN ? ahead + (float)(k - k_ref) : ahead;
+    if (__builtin_amdgcn_ballot_w64(level > kMaxAhead) != 0) {
       float alpha = 1.f;
-      if (ahead > kMaxAhead) {
+      if (ahead > 0.f) {
         alpha = fast_exp2(m_ref - mx);  // exp2(-inf) = 0 on the first visible step
         m_ref = mx;
         m_ref_safe = mx;
@@ -346,12 +358,12 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
       for (int db = 0; db < 8; ++db) acc[db] *= alpha;
     }
     // n: whole powers of two from the reference up (or down) to this step's maximum
-    const float nf = __builtin_ceilf(fmaxf(ahead, -kMaxAhead));  // (NaN, -inf: no visible key; every P is 0)
+    const float nf = __builtin_ceilf(fmaxf(ahead, -kMaxBehind));  // (NaN, -inf: no visible key; every P is 0)
     const int n = (int)nf;
     const float e_add = (float)(kPBits - k) - m_ref_safe - nf;
-    // E8M0 block scale of P, 2^(p_scale - 127); n and k - k_ref are at most kMaxAhead each
+    // E8M0 block scale of P, 2^(p_scale - 127): n + (k - k_ref) is at most kMaxAhead + 1; 255 would be a NaN
     int p_scale = n + (127 + k - k_ref);
-    p_scale = p_scale < 1 ? 1 : p_scale;
+    p_scale = p_scale < 1 ? 1 : (p_scale > 254 ? 254 : p_scale);
     const float e_mul = FULL ? rscale : 1.f;
     float psum = 0.f;
     uint32_t ph[4] = {0u, 0u, 0u, 0u}, pl[4] = {0u, 0u, 0u, 0u};  // (HALF: the tiles that are not this wave's hold P = 0)

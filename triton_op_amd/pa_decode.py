@@ -8,8 +8,12 @@ pa_decode_triton.py:523-685.  Differences, all additive:
 
 * `query` may be bf16 (no `query_scale`) as well as FP8 e4m3fn with a per-tensor or per-token scale;
 * the caches may be bf16 (no scales) as well as FP8 with per-tensor (0-dim) or per-token scales;
-* the partition buffers can be passed in (`exp_sums`, `max_logits`, `tmp_output`), in which case
-  nothing is allocated;
+* the partition buffers can be passed in, in which case nothing is allocated: `max_logits`, `exp_sums`,
+  `tmp_output` (or `temp_output`) follow `alibi_slopes`, positionally or by keyword, as in the reference's harness
+  wrappers (test_pa_mtp.py:566-584 run_gluon_fp8_kernel, test_pa_decode_gluon_triton.py:264-297 run_triton, which
+  accept and ignore them);
+* `alibi_slopes` holds one slope per packed query row ([num_kv_heads * query_sequence_length * group], what the
+  reference kernels index, :323-327) or one per query head ([num_kv_heads * group]);
 * `partition_size` may be any multiple of 256 (the reference's constant); by default the tuning
   layer picks it from the batch shape and the longest context;
 * `query_lens` gives a per-sequence number of new tokens (ragged MTP batches);
@@ -125,16 +129,21 @@ def plan_decode(
     value_scale: Optional[torch.Tensor] = None,
     num_sequence_partitions: int = 0,
     alibi_slopes: Optional[torch.Tensor] = None,
-    *,
-    exp_sums: Optional[torch.Tensor] = None,
     max_logits: Optional[torch.Tensor] = None,
+    exp_sums: Optional[torch.Tensor] = None,
     tmp_output: Optional[torch.Tensor] = None,
+    *,
+    temp_output: Optional[torch.Tensor] = None,
     partition_size: Optional[int] = None,
     query_lens: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
     sinks: Optional[torch.Tensor] = None,
     reuse_item_list: bool = False,
 ) -> DecodePlan:
+    if temp_output is not None:  # the spelling of run_gluon_fp8_kernel (test_pa_mtp.py:566-584)
+        if tmp_output is not None and tmp_output is not temp_output:
+            raise ValueError("tmp_output and temp_output name the same buffer: pass one of them")
+        tmp_output = temp_output
     # ---- shapes (pa_decode_triton_gluon_fp8.py:1703-1722) ------------------------------------
     if output.dim() != 3:
         raise ValueError(f"Expected 3D output tensor, but got shape {tuple(output.shape)}")
@@ -248,8 +257,12 @@ def plan_decode(
     elif (key_scale is None) != (value_scale is None):
         raise ValueError("key_scale and value_scale must be given together")
     if alibi_slopes is not None:
-        if alibi_slopes.dtype != torch.float32 or alibi_slopes.numel() != num_kv_heads * group or not alibi_slopes.is_contiguous():
-            raise ValueError(f"alibi_slopes must be contiguous float32 [{num_kv_heads * group}]")
+        # one slope per packed query row, [num_kv_heads * query_sequence_length * group] at h*Ge + t*G + g: the array the
+        # reference kernels index (:323-327, :803-810); or one per query head, [num_kv_heads * group]
+        if alibi_slopes.dtype != torch.float32 or not alibi_slopes.is_contiguous() or \
+                alibi_slopes.numel() not in (rows_total, num_kv_heads * group):
+            raise ValueError(f"alibi_slopes must be contiguous float32 [{rows_total}] (one slope per query row) "
+                             f"or [{num_kv_heads * group}] (one per query head)")
     if sinks is not None:
         if sinks.dtype != torch.float32 or sinks.numel() != rows_total or not sinks.is_contiguous() or sinks.device != dev:
             raise ValueError(f"sinks must be contiguous float32 [{rows_total}] (one logit per query row) on {dev}")
@@ -323,6 +336,7 @@ def plan_decode(
     a.key_scale = _ptr(key_scale) if kv_mode != _cabi.PA_QUANT_NONE else None
     a.value_scale = _ptr(value_scale) if kv_mode != _cabi.PA_QUANT_NONE else None
     a.alibi_slopes = _ptr(alibi_slopes)
+    a.alibi_slopes_len = 0 if alibi_slopes is None else alibi_slopes.numel()
     a.sinks = _ptr(sinks)
     a.exp_sums, a.max_logits, a.tmp_output = exp_sums.data_ptr(), max_logits.data_ptr(), tmp_output.data_ptr()
     # zeroed work-item counter for ragged batches (the kernels leave it zero, so the plan can be replayed) plus
@@ -374,10 +388,11 @@ def paged_attention_decode(
     value_scale: Optional[torch.Tensor] = None,
     num_sequence_partitions: int = 0,
     alibi_slopes: Optional[torch.Tensor] = None,
-    *,
-    exp_sums: Optional[torch.Tensor] = None,
     max_logits: Optional[torch.Tensor] = None,
+    exp_sums: Optional[torch.Tensor] = None,
     tmp_output: Optional[torch.Tensor] = None,
+    *,
+    temp_output: Optional[torch.Tensor] = None,
     partition_size: Optional[int] = None,
     query_lens: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
@@ -389,8 +404,8 @@ def paged_attention_decode(
     plan = plan_decode(
         output, query, key_cache, value_cache, sequence_lengths, block_tables, softmax_scale,
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
-        num_sequence_partitions, alibi_slopes, exp_sums=exp_sums, max_logits=max_logits,
-        tmp_output=tmp_output, partition_size=partition_size, query_lens=query_lens, workspace=workspace,
+        num_sequence_partitions, alibi_slopes, max_logits, exp_sums, tmp_output, temp_output=temp_output,
+        partition_size=partition_size, query_lens=query_lens, workspace=workspace,
         sinks=sinks, reuse_item_list=reuse_item_list)
     plan.run()
     return {

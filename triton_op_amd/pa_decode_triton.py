@@ -24,10 +24,10 @@ def paged_attention_decode(
     v_scale: Optional[torch.Tensor] = None,
     num_seq_partitions: int = 0,
     alibi_slopes: Optional[torch.Tensor] = None,
-    *,
+    max_logits: Optional[torch.Tensor] = None,   # trailing positions of run_triton (test_pa_decode_gluon_triton.py:264-281)
     exp_sums: Optional[torch.Tensor] = None,
-    max_logits: Optional[torch.Tensor] = None,
     tmp_output: Optional[torch.Tensor] = None,
+    *,
     partition_size: Optional[int] = None,
 ) -> Dict[str, object]:
     # The reference reads the scalar scales with .item() (a host sync per call, :619-620); here the
@@ -36,8 +36,8 @@ def paged_attention_decode(
         k_scale = v_scale = None
     res = _impl.paged_attention_decode(
         output, query, key_cache, value_cache, seq_lens, block_tables, attn_scale, 1, max_seq_len,
-        compute_type, None, k_scale, v_scale, num_seq_partitions, alibi_slopes,
-        exp_sums=exp_sums, max_logits=max_logits, tmp_output=tmp_output, partition_size=partition_size)
+        compute_type, None, k_scale, v_scale, num_seq_partitions, alibi_slopes, max_logits, exp_sums, tmp_output,
+        partition_size=partition_size)
     return {
         "tmp_output": res["temporary_output"],
         "exp_sums": res["exponential_sums"],
