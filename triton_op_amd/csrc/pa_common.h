@@ -23,6 +23,8 @@ constexpr int kHeadSize = 128;
 // PaDecodeArgs.flags as the kernels see it (the launch layer sets it in its own copy of the arguments)
 constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning kernel's item list
 constexpr int kFlagSpanShift = 20;         // bits 20..27: partitions a one-wave workgroup walks in one pass (0 = 1)
+// experiment switch of pa_partition_shared_kernel: P without its FP8 residual
+constexpr int kFlagResidualNever = 0x40000;
 constexpr int kSpanMax = 4;                // ... at most (their partial results wait in LDS for the end of the pass)
 // Workspace layout (int32 words): [0], [1] counters of the queued launch, [2] number of listed items,
 // [16 + 2i], [17 + 2i] sequence and partition index of item i.

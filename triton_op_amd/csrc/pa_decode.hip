@@ -82,6 +82,7 @@ int device_num_cus() {
 //   PA_DECODE_QUEUE=0    no queued launch          PA_DECODE_SHARED=0   one workgroup per 16-row tile, always
 //   PA_DECODE_SORTED=0|1 never / always the sorted dispatch (when the workspace has room)
 //   PA_DECODE_LDS_PAD=n  unused LDS per workgroup of the shared-stream kernel (lowers its occupancy)
+//   PA_DECODE_P_RESIDUAL=0  shared-stream kernel: P without its FP8 residual (every element rounded to e4m3)
 // All are read once, at the first launch.
 int debug_switch(const char* name, int unset) {
   static const bool enabled = [] {
@@ -275,6 +276,10 @@ int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t s
     k.flags = kFlagSortedItems;
   }
   if (c.span > 1) k.flags |= c.span << kFlagSpanShift;
+  // experiment (PA_DECODE_DEBUG=1): PA_DECODE_P_RESIDUAL=0 drops the FP8 residual of P in the shared-stream kernel
+  // (every P rounded to e4m3, as the reference's kernel rounds it)
+  static const int p_residual = debug_switch("PA_DECODE_P_RESIDUAL", 1);
+  if (p_residual == 0) k.flags |= kFlagResidualNever;
   if (!c.fp8) {
     if (c.row_tiles == 2) return launch_partition_tile<2, PA_DTYPE_BF16, false, false>(k, c, stream);
     return launch_partition_tile<1, PA_DTYPE_BF16, false, false>(k, c, stream);
