@@ -420,8 +420,14 @@ def test_launch_layer_choices(pa_lib):
     assert "queued items" in info(b=64, hq=128, hkv=8, q=4, ctx=4096, ps=4096, kv="bf16", ragged=True)
     assert "queued items" not in info(b=64, hq=128, hkv=8, q=4, ctx=4096, ps=4096, kv="bf16", ragged=True, workspace=False)
     # more sequences than the item tables of the queued / sorted launches hold: plain order, no error
+    # (a tile of up to 8 real rows stages half the bytes per partition: up to eight partitions per workgroup)
     assert info(b=5000, hq=8, hkv=1, q=1, ctx=4096, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 10000, 8 partitions per workgroup"
+    assert info(b=5000, hq=16, hkv=1, q=1, ctx=4096, ps=256) == \
         "pa_partition_kernel<fp8, bs16, 1 waves> x 20000, 4 partitions per workgroup"
+    # c4 at the reference's partition size: 512 partitions per sequence, eight per workgroup, one round
+    assert info(b=4, hq=64, hkv=8, q=1, ctx=131072, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 8 partitions per workgroup"
     # bad arguments are refused as by the launch itself
     a = _fake_args(b=4, hq=8, hkv=1, q=1, ctx=1024, ps=300)
     assert pa_lib.pa_decode_launch_info(C.byref(a), C.create_string_buffer(64), 64) == -4

@@ -389,13 +389,17 @@ def test_sorted_dispatch_of_a_many_round_launch(cuda, group, q_len, scale_mode):
     torch.testing.assert_close(outs[0].float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
 
 
-@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span,alibi,batch",
-                         [("fp8", "tensor", 2, 1, False, 16, 256, 3, False, 200), ("fp8", "token", 4, 2, False, 16, 256, 3, False, 200),
-                          ("fp8", "tensor", 8, 2, False, 64, 256, 3, False, 200), ("fp8", "tensor", 8, 2, False, 1024, 512, 2, False, 200),
-                          ("bf16", "none", 16, 4, True, 16, 256, 4, False, 200), ("fp8", "token", 8, 1, False, 16, 256, 3, True, 200),
+@pytest.mark.parametrize("kv,scale_mode,group,q_len,ragged,block_size,ps,span,alibi,batch,max_ctx",
+                         [("fp8", "tensor", 2, 1, False, 16, 256, 3, False, 200, 1100), ("fp8", "token", 4, 2, False, 16, 256, 3, False, 200, 1100),
+                          ("fp8", "tensor", 8, 2, False, 64, 256, 3, False, 200, 1100), ("fp8", "tensor", 8, 2, False, 1024, 512, 2, False, 200, 1100),
+                          ("bf16", "none", 16, 4, True, 16, 256, 4, False, 200, 1100), ("fp8", "token", 8, 1, False, 16, 256, 3, True, 200, 1100),
                           # 600 x 8 x ceil(5 / 4) coarse items are more than two rounds: the walk AND the sorted dispatch
-                          ("fp8", "tensor", 8, 1, False, 16, 256, 4, False, 600), ("fp8", "token", 4, 2, False, 16, 256, 4, True, 600)])
-def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span, alibi, batch):
+                          # (8 rows per kv head: half-size slots, all five partitions in one workgroup)
+                          ("fp8", "tensor", 8, 1, False, 16, 256, 5, False, 600, 1100), ("fp8", "token", 4, 2, False, 16, 256, 5, True, 600, 1100),
+                          ("fp8", "tensor", 16, 1, False, 16, 256, 4, False, 600, 1100),
+                          # nine partitions, eight rows: eight partitions per workgroup, then one
+                          ("fp8", "tensor", 8, 1, False, 16, 256, 8, False, 400, 2100), ("fp8", "token", 2, 3, False, 16, 256, 8, True, 400, 2100)])
+def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_len, ragged, block_size, ps, span, alibi, batch, max_ctx):
     """A caller-fixed small partition size and several rounds of one-wave workgroups: every workgroup then walks
     several consecutive partitions in one pass over the pages (the launch layer says so) and writes one partial
     result per partition.  The partition buffers are held against the oracle's partition stage, the merged result
@@ -411,8 +415,8 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     from triton_op_amd import _cabi
 
     gen = torch.Generator().manual_seed(33)
-    ctx = torch.randint(1, 1101, (batch,), generator=gen, dtype=torch.int32)
-    ctx[:9] = torch.tensor([1, 255, 256, 257, 512, 768, 769, 1024, 1100], dtype=torch.int32)
+    ctx = torch.randint(1, max_ctx + 1, (batch,), generator=gen, dtype=torch.int32)
+    ctx[:9] = torch.tensor([1, 255, 256, 257, 512, 768, 769, 1024, max_ctx], dtype=torch.int32)
     ctx = torch.clamp(ctx, min=q_len)
     q_lens = None
     if ragged:
@@ -420,7 +424,7 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
         q_lens[:4] = torch.tensor([1, q_len, 2, 1], dtype=torch.int32)
     wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, q_lens=q_lens,
                kv_dtype=kv, scale_mode=scale_mode, block_size=block_size)
-    sorted_too = batch == 600
+    sorted_too = batch >= 400
     if sorted_too:  # an empty sequence among them (the generator wants a page per sequence: declared empty afterwards)
         ctx = ctx.clone()
         ctx[11] = 0
@@ -430,9 +434,9 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     out = torch.full_like(g.query, float("nan"))
     slopes = torch.linspace(0.01, 0.3, wl.query.shape[1], dtype=torch.float32) if alibi else None
     plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
-                         q_len, 1100, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
+                         q_len, max_ctx, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
                          query_lens=g.q_lens, alibi_slopes=None if slopes is None else slopes.to(cuda))
-    P = -(-1100 // ps)
+    P = -(-max_ctx // ps)
     assert plan.args.max_num_partitions == P
     if ragged:
         plan.args.workspace = None
@@ -827,3 +831,46 @@ def test_adversarial_softmax_levels(cuda, kind, rows):
         assert bool(torch.isfinite(gto[reach[..., None].expand_as(to)]).all())
         sel = reach[..., None].expand_as(to)
         torch.testing.assert_close((gto / tmag)[sel], (to / tmag)[sel], atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("group,q_len,ragged,with_sinks", [(8, 1, False, False), (6, 4, True, False), (8, 3, False, True),
+                                                          (16, 2, True, True)])
+def test_many_partitions_of_few_rows_take_the_wide_reduce(cuda, group, q_len, ragged, with_sinks):
+    """A handful of long sequences at the reference's 256-token partitions: few 16-row units with 64 partitions or
+    more each go to the reduce kernel whose workgroup splits the partition axis over its sixteen waves.  In the
+    batch: 79 and 67 partitions, two partitions, one partition (finished by the partition kernel: the merge must
+    leave its rows alone in pa_decode and reproduce them in pa_decode_reduce), an empty sequence; 8, 24, 24 and 32
+    rows per kv head (units of 8 and 16 rows, padding rows of a ragged batch, rows of padding query positions)."""
+    import triton_op_amd as T
+
+    ctx = _ctx(20000, 300, 17000, 100, q_len)
+    q_lens = _ctx(q_len, 1, max(1, q_len - 1), q_len, 1) if ragged else None
+    wl = _make(batch=5, num_q_heads=group * 2, num_kv_heads=2, context_lens=ctx, q_len=q_len, q_lens=q_lens, seed=29)
+    ctx0 = ctx.clone()
+    ctx0[4] = 0  # declared empty after the generator gave it a page
+    wl = type(wl)(**{**wl.__dict__, "context_lens": ctx0})
+    g = wl.to(cuda)
+    sinks = torch.linspace(-2.0, 3.0, wl.query.shape[1], dtype=torch.float32) if with_sinks else None
+    out = torch.full_like(g.query, float("nan"))
+    plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale, q_len,
+                         20000, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=256, query_lens=g.q_lens,
+                         sinks=None if sinks is None else sinks.to(cuda))
+    assert plan.args.max_num_partitions == 79
+    plan.run()
+    torch.cuda.synchronize()
+    live = [0, 1, 2, 3]
+    ref = O.paged_attention_decode_oracle(wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                                          wl.softmax_scale, q_len if q_lens is None else q_lens, wl.key_scale, wl.value_scale,
+                                          seq_ids=live, sinks=sinks, q_max=q_len)
+    assert not torch.isnan(out.float()).any()
+    assert bool((out[4] == 0).all())
+    torch.testing.assert_close(out.float().cpu()[live], ref.float()[live], atol=ATOL, rtol=RTOL)
+    # the merge alone (every sequence, also the one-partition one) on the kernel's own buffers against the closed form
+    first = out.clone()
+    out.fill_(float("nan"))
+    plan.run_reduce()
+    torch.cuda.synchronize()
+    if sinks is None:
+        merged = O.reduce_stage(plan.max_logits.cpu(), plan.exp_sums.cpu(), plan.tmp_output.float().cpu(), wl.context_lens, 256)
+        torch.testing.assert_close(out.float().cpu(), merged.float(), atol=4e-3, rtol=8e-3)  # bf16 rounding only
+    torch.testing.assert_close(out.float().cpu(), first.float().cpu(), atol=4e-3, rtol=8e-3)

@@ -25,7 +25,10 @@ constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning k
 constexpr int kFlagSpanShift = 20;         // bits 20..27: partitions a one-wave workgroup walks in one pass (0 = 1)
 // experiment switch of pa_partition_shared_kernel: P without its FP8 residual
 constexpr int kFlagResidualNever = 0x40000;
-constexpr int kSpanMax = 4;                // ... at most (their partial results wait in LDS for the end of the pass)
+// ... at most: their partial results wait in LDS for the end of the pass, in a pool of kSpanPoolBytes per 16-row
+// tile; a tile of up to 8 real rows stages only those (half the bytes) and may walk twice as many partitions
+constexpr int kSpanMax = 4;
+constexpr int kSpanMaxFewRows = 8;
 // Workspace layout (int32 words): [0], [1] counters of the queued launch, [2] number of listed items,
 // [16 + 2i], [17 + 2i] sequence and partition index of item i.
 constexpr int kPlanHeaderWords = 16;
@@ -158,8 +161,10 @@ __device__ __forceinline__ u32x4 keep_first_bytes(u32x4 v, int n) {
 // rows of the partial output.  The tile is transposed through a wave-private LDS buffer so that every
 // store instruction writes four whole 256-byte rows (16 bytes per lane) instead of 32-byte fragments.
 constexpr int kORowBytes = 272;  // 256 B of bf16 + 16 B pad
-// first half: the tile, scaled and rounded to bf16, into the LDS buffer (row li at li * kORowBytes)
-__device__ __forceinline__ void stage_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, int lane) {
+constexpr int kSpanPoolBytes = kSpanMaxFewRows * (8 * kORowBytes + 2 * 16 * 4);  // >= kSpanMax slots of 16 rows
+// first half: the tile, scaled and rounded to bf16, into the LDS buffer (row li at li * kORowBytes); only the first
+// `rows` rows are staged (the buffer may be no longer than that)
+__device__ __forceinline__ void stage_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, int lane, int rows = 16) {
   const int li = lane & 15, kg = lane >> 4;
 #pragma unroll
   for (int db = 0; db < 8; ++db) {
@@ -167,7 +172,7 @@ __device__ __forceinline__ void stage_partial_tile(char* lds, const f32x4 (&acc)
     u32x2 pk;
     pk[0] = pack_bf16x2(o[0], o[1]);
     pk[1] = pack_bf16x2(o[2], o[3]);
-    *reinterpret_cast<u32x2*>(lds + li * kORowBytes + (16 * db + 4 * kg) * 2) = pk;
+    if (li < rows) *reinterpret_cast<u32x2*>(lds + li * kORowBytes + (16 * db + 4 * kg) * 2) = pk;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -180,8 +185,8 @@ __device__ __forceinline__ void copy_staged_tile(const char* lds, char* dst, int
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = 4 * i + kg;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(lds + r * kORowBytes + li * 16);
-    if (r < rows_to_write) {
+    if (r < rows_to_write) {  // (rows at or beyond may not exist in the buffer)
+      const u32x4 v = *reinterpret_cast<const u32x4*>(lds + r * kORowBytes + li * 16);
       *reinterpret_cast<u32x4*>(dst + (int64_t)r * row_stride_bytes + li * 16) = v;
       if (dst2) *reinterpret_cast<u32x4*>(dst2 + (int64_t)r * row_stride2_bytes + li * 16) = v;
     }
@@ -191,8 +196,8 @@ __device__ __forceinline__ void copy_staged_tile(const char* lds, char* dst, int
 }
 __device__ __forceinline__ void store_partial_tile(char* lds, const f32x4 (&acc)[8], float inv, char* dst,
                                                    int64_t row_stride_bytes, char* dst2, int64_t row_stride2_bytes,
-                                                   int rows_to_write, int lane) {
-  stage_partial_tile(lds, acc, inv, lane);
+                                                   int rows_to_write, int lane, int rows_staged = 16) {
+  stage_partial_tile(lds, acc, inv, lane, rows_staged);
   copy_staged_tile(lds, dst, row_stride_bytes, dst2, row_stride2_bytes, rows_to_write, lane);
 }
 

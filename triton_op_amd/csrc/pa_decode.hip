@@ -206,7 +206,9 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     if (a.block_size > 64 && a.partition_size < 512) span = 1;
     if (forced_span > 0) span = forced_span;
     span = span > a.max_num_partitions ? a.max_num_partitions : span;
-    span = span > kSpanMax ? kSpanMax : span;
+    // (a tile of up to 8 real rows stages half the bytes per partition and may walk twice as many)
+    const long long span_max = c.row_tiles == 1 && ge <= 8 ? kSpanMaxFewRows : kSpanMax;
+    span = span > span_max ? span_max : span;
     if (span >= 2) {
       c.span = (int)span;
       const long long coarse = (a.max_num_partitions + span - 1) / span;
@@ -353,6 +355,15 @@ int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
   // enough rows to fill the GPU's wave slots several times over: four rows per wave
   const bool big = blocks * 16 >= 16384;
   const dim3 grid((unsigned)blocks);
+  // Few 16-row units, many partitions each (a caller-fixed small partition size on a handful of long sequences): a
+  // unit is cut along the head dimension into several workgroups, whose waves split the partition axis.  Needs
+  // 16-byte aligned rows of tmp_output.
+  if (blocks <= 2LL * device_num_cus() && a->max_num_partitions >= 64 && (a->stride_tmp_g * 2) % 16 == 0 &&
+      (a->stride_tmp_p * 2) % 16 == 0 && (a->stride_tmp_h * 2) % 16 == 0 && (a->stride_tmp_s * 2) % 16 == 0 &&
+      (reinterpret_cast<uintptr_t>(a->tmp_output) & 15) == 0)
+    return skip_single
+               ? pa_launch(pa_reduce_wide_kernel<true>, dim3((unsigned)blocks * kWideDimSplit), dim3(64 * kWideWaves), 0, stream, *a)
+               : pa_launch(pa_reduce_wide_kernel<false>, dim3((unsigned)blocks * kWideDimSplit), dim3(64 * kWideWaves), 0, stream, *a);
   if (skip_single)
     return big ? pa_launch(pa_reduce_kernel<true, 4>, grid, dim3(256), 0, stream, *a)
                : pa_launch(pa_reduce_kernel<true, 1>, grid, dim3(1024), 0, stream, *a);

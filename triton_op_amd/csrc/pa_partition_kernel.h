@@ -64,13 +64,13 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   typedef StepData<KVT, PER_TOKEN> SD;
 
   __shared__ __attribute__((aligned(16))) char p_lds[FP8MATH ? 1 : WAVES][FP8MATH ? 1 : NT][FP8MATH ? 16 : 16 * kPRowBytes];
-  __shared__ __attribute__((aligned(16))) char o_lds[1][16 * kORowBytes];
-  // SPAN: the partial results of the partitions a workgroup has left behind wait here for the end of the pass
-  // (stores in the middle of the page stream would hold up the loads issued after them: memory operations of a
-  // wave retire in order).  Per partition and row tile: 16 staged bf16 rows, then 16 maxima and 16 sums.
-  constexpr int kSpanSlotBytes = 16 * kORowBytes + 2 * 16 * 4;
+  // SPAN: the partial results of the partitions a workgroup walks wait here for the end of the pass (stores in the
+  // middle of the page stream would hold up the loads issued after them: memory operations of a wave retire in
+  // order), the last partition's included.  Per partition and row tile: the staged bf16 rows (16, or 8 when the
+  // tile has no more real rows than that: half the bytes, twice the partitions), then 16 maxima and 16 sums.
   constexpr bool kSpanCapable = WAVES == 1 && !QUEUE;
-  __shared__ __attribute__((aligned(16))) char span_lds[kSpanCapable ? (kSpanMax - 1) * NT * kSpanSlotBytes : 16];
+  __shared__ __attribute__((aligned(16))) char o_lds[1][kSpanCapable ? 16 : 16 * kORowBytes];
+  __shared__ __attribute__((aligned(16))) char span_lds[kSpanCapable ? NT * kSpanPoolBytes : 16];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -131,11 +131,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // over the pages, and writes the partial result of each as it crosses into the next.  For callers whose buffers
   // fix a small partition size (the reference's constant 256): the query set-up and the ramp of the page stream
   // are paid once per span instead of once per four steps.
+  // rows staged per tile and the bytes of a tile's slot in the pool
+  const int span_rows = (NT == 1 && Ge <= 8) ? 8 : 16;
+  const int span_slot_bytes = span_rows * kORowBytes + 2 * 16 * 4;
   int span = 1;
   if constexpr (kSpanCapable) {
+    const int span_max = span_rows == 8 ? kSpanMaxFewRows : kSpanMax;
     span = (a.flags >> kFlagSpanShift) & 0xff;
-    span = span < 1 ? 1 : (span > kSpanMax ? kSpanMax : span);
+    span = span < 1 ? 1 : (span > span_max ? span_max : span);
   }
+  static_assert(kSpanMax * (16 * kORowBytes + 2 * 16 * 4) <= kSpanPoolBytes, "the pool holds kSpanMax full tiles");
 
   for (;;) {  // one pass without the queue
   int h, rt, b, part, tiles_b = RT;
@@ -716,7 +721,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run[nt] : 1.f) * (1.f / 256.f) : 1.f;
-          char* slot = &span_lds[0] + ((part_cur - part) * NT + nt) * kSpanSlotBytes;
+          char* slot = &span_lds[0] + ((part_cur - part) * NT + nt) * span_slot_bytes;
           float l_tot = quad_row_sum(l_run[nt]);
           float m_out = m_run[nt];
           if (row0 + 16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
@@ -725,10 +730,10 @@ void pa_partition_kernel(const PaDecodeArgs a) {
           }
           const float inv = l_tot > 0.f ? v_tensor_scale * acc_unit / l_tot : 0.f;
           if (kg == 0) {
-            reinterpret_cast<float*>(slot + 16 * kORowBytes)[li] = m_out * (1.0f / kLog2e);
-            reinterpret_cast<float*>(slot + 16 * kORowBytes)[16 + li] = l_tot;
+            reinterpret_cast<float*>(slot + span_rows * kORowBytes)[li] = m_out * (1.0f / kLog2e);
+            reinterpret_cast<float*>(slot + span_rows * kORowBytes)[16 + li] = l_tot;
           }
-          stage_partial_tile(slot, acc[nt], inv, lane);
+          stage_partial_tile(slot, acc[nt], inv, lane, span_rows);
         }
         reset_state();
         ++part_cur;
@@ -803,9 +808,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         a.max_logits[es_off + row] = m_run[nt] * (1.0f / kLog2e);
         a.exp_sums[es_off + row] = l_tot[nt];
       }
-      store_partial_tile(&o_lds[0][0], acc[nt], inv, tmp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2,
+      // (one-wave workgroups stage the last partition's tile in the next free slot of the pool)
+      char* stage_at = kSpanCapable ? &span_lds[0] + ((part_cur - part) * NT + nt) * span_slot_bytes : &o_lds[0][0];
+      store_partial_tile(stage_at, acc[nt], inv, tmp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2,
                          a.stride_tmp_g * 2, direct ? outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2 : nullptr,
-                         a.stride_out_h * 2, Ge - row0 - 16 * nt, lane);
+                         a.stride_out_h * 2, Ge - row0 - 16 * nt, lane, kSpanCapable ? span_rows : 16);
     }
   } else {
     // merge the waves' (m, l, O): every wave holds the same (row, head dim) in the same lane and register,
@@ -878,11 +885,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
                                         (int64_t)pc * a.stride_tmp_p) * 2;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const char* slot = &span_lds[0] + ((pc - part) * NT + nt) * kSpanSlotBytes;
+        const char* slot = &span_lds[0] + ((pc - part) * NT + nt) * span_slot_bytes;
         const int row = row0 + 16 * nt + li;
         if (row < Ge && kg == 0) {
-          a.max_logits[eo + row] = reinterpret_cast<const float*>(slot + 16 * kORowBytes)[li];
-          a.exp_sums[eo + row] = reinterpret_cast<const float*>(slot + 16 * kORowBytes)[16 + li];
+          a.max_logits[eo + row] = reinterpret_cast<const float*>(slot + span_rows * kORowBytes)[li];
+          a.exp_sums[eo + row] = reinterpret_cast<const float*>(slot + span_rows * kORowBytes)[16 + li];
         }
         copy_staged_tile(slot, tp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2, a.stride_tmp_g * 2, nullptr, 0,
                          Ge - row0 - 16 * nt, lane);

@@ -194,6 +194,133 @@ __global__ __launch_bounds__(1024 / ROWS) void pa_reduce_listed_kernel(const PaD
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The merge of MANY partitions for FEW rows (a handful of very long sequences cut into the reference's 256-token
+// partitions: 4 sequences x 8 kv heads x 512 partitions).  pa_reduce_kernel gives such a call one wave per output
+// row, which walks the row's partitions one after the other: 32 workgroups of 8 busy waves on 32 of the GPU's
+// CUs, each wave waiting for its own chain of loads, and a CU can take in only so many bytes per cycle.  Here a
+// 16-row unit is cut along the HEAD DIMENSION into kWideDimSplit workgroups (no exchange between them: their
+// output columns are disjoint), and inside a workgroup the sixteen waves split the PARTITION axis into
+// interleaved streams: one 16-byte load per lane fetches eight head dims of one row, a wave's load
+// instruction covers all sixteen rows of kWideParts partitions (two partitions of a unit with at most eight rows),
+// eight such loads go out before anything is waited for.
+//   phase A  M[row] = max over the partitions of max_logits                  (lanes: row, partition slot)
+//   phase B  acc += exp_sums * exp(max_logits - M) * partial                  (lanes: row, 8 head dims)
+//   phase C  the waves' acc and sums of the weights meet in LDS; a thread owns one head dim of one row
+// ---------------------------------------------------------------------------------------------
+constexpr int kWideWaves = 16;
+constexpr int kWideDimSplit = 4;                          // workgroups per 16-row unit
+constexpr int kWideDims = kHeadSize / kWideDimSplit;      // head dims of one workgroup
+constexpr int kWideRowLanes = kWideDims / 8;              // lanes that share a row (eight head dims each)
+constexpr int kWideParts = 64 / (16 * kWideRowLanes);     // partitions one load instruction of a wave covers (16-row unit)
+constexpr int kWideStreamsMax = kWideWaves * kWideParts * 2;  // ... twice as many when the unit has at most 8 rows
+static_assert(kWideRowLanes >= 1 && kWideParts >= 1 && kWideParts * 16 * kWideRowLanes == 64, "lane map of the wide reduce");
+template <bool SKIP_SINGLE>
+__global__ __launch_bounds__(64 * kWideWaves) void pa_reduce_wide_kernel(const PaDecodeArgs a) {
+  __shared__ float s_max[kWideStreamsMax][16];
+  __shared__ float s_sum[kWideStreamsMax][16];
+  __shared__ float s_acc[kWideStreamsMax][16][kWideDims + 4];  // a stream's partial results (rows padded against bank conflicts)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int Ge = a.q_len * a.group_size;
+  const int RT = (Ge + 15) / 16;
+  long long wid = blockIdx.x;
+  const int chunk = (int)(wid % kWideDimSplit);
+  wid /= kWideDimSplit;
+  const int rt = (int)(wid % RT);
+  const int h = (int)((wid / RT) % a.num_kv_heads);
+  const int b = (int)(wid / ((long long)RT * a.num_kv_heads));
+  const int row0 = 16 * rt;
+
+  const int ctx = sload_i32(a.context_lens + b);
+  int n = (ctx + a.partition_size - 1) / a.partition_size;
+  n = n > a.max_num_partitions ? a.max_num_partitions : n;
+  if (SKIP_SINGLE && n == 1 && !a.sinks) return;  // the partition kernel has written these rows
+  const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
+  const int rows_valid = n <= 0 ? 0 : qb * a.group_size;     // rows at or beyond read as zero
+  const int rows_here = min(16, Ge - row0);                  // rows of this unit that exist in the buffers
+  const int rows_live = max(0, min(16, rows_valid - row0));  // ... and hold a result
+  // this lane's partition stream, its row of the unit and its eight head dims of the chunk: a unit of at most 8 rows
+  // gives the lanes of rows 8..15 a second partition instead (partition p belongs to stream p % streams)
+  const int row_bits = rows_here <= 8 ? 3 : 4;
+  const int dl = lane % kWideRowLanes, r = (lane / kWideRowLanes) & ((1 << row_bits) - 1), pp = lane / (kWideRowLanes << row_bits);
+  const int parts = 64 / (kWideRowLanes << row_bits);
+  const int streams = kWideWaves * parts;
+  const int stream = wave * parts + pp;
+  const bool live = r < rows_live;
+
+  const int64_t sp = a.stride_es_p;
+  const float* ml = a.max_logits + (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + row0 + (live ? r : 0);
+  const float* es = a.exp_sums + (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + row0 + (live ? r : 0);
+  const char* tmp = (const char*)a.tmp_output +
+                    ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h + (int64_t)(row0 + (live ? r : 0)) * a.stride_tmp_g) * 2 +
+                    (chunk * kWideDims + 8 * dl) * 2;
+  const int64_t tp = a.stride_tmp_p * 2;
+
+  // ---- phase A: the lanes of a row walk the stream's partitions in turn
+  float M = -INFINITY;
+  if (live)
+    for (int p = stream + streams * dl; p < n; p += kWideRowLanes * streams) M = fmaxf(M, ml[(int64_t)p * sp]);
+#pragma unroll
+  for (int o = 1; o < kWideRowLanes; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
+  if (dl == 0) s_max[stream][r] = M;
+  __syncthreads();
+  M = s_max[0][r];
+  for (int w = 1; w < streams; ++w) M = fmaxf(M, s_max[w][r]);
+  const float M_safe = M == -INFINITY ? 0.f : M;
+
+  // ---- phase B: this stream's partitions, eight at a time; every load of a batch goes out first
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float wsum = 0.f;
+  for (int p0 = stream; p0 - pp < n; p0 += 8 * streams) {  // (the lanes of a wave leave together)
+    float m[8], l[8];
+    u32x4 t[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int p = p0 + streams * q;
+      const bool on = live && p < n;
+      const int pc = p < n ? p : 0;  // (an address inside the buffers for the lanes that load nothing real)
+      m[q] = on ? ml[(int64_t)pc * sp] : -INFINITY;
+      l[q] = on ? es[(int64_t)pc * sp] : 0.f;
+      t[q] = on ? load16(tmp + (int64_t)pc * tp) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float w = l[q] > 0.f ? l[q] * __expf(m[q] - M_safe) : 0.f;
+      wsum += w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] += bf16_bits_to_f32(t[q][e] & 0xffffu) * w;
+        acc[2 * e + 1] += __uint_as_float(t[q][e] & 0xffff0000u) * w;
+      }
+    }
+  }
+
+  // ---- phase C: the streams' sums meet in LDS (the lanes of a row hold the same sum of weights)
+  if (dl == 0) s_sum[stream][r] = wsum;
+  *reinterpret_cast<f32x4*>(&s_acc[stream][r][8 * dl]) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+  *reinterpret_cast<f32x4*>(&s_acc[stream][r][8 * dl + 4]) = f32x4{acc[4], acc[5], acc[6], acc[7]};
+  __syncthreads();
+  // thread t < 16 * kWideDims: row t / kWideDims, head dim t % kWideDims of the chunk
+  const int row = (int)threadIdx.x / kWideDims, d = (int)threadIdx.x % kWideDims;
+  if (threadIdx.x >= 16 * kWideDims || row >= rows_here) return;
+  float o = 0.f, tot = 0.f;
+  for (int w = 0; w < streams; ++w) {
+    o += s_acc[w][row][d];
+    tot += s_sum[w][row];
+  }
+  float Mr = s_max[0][row];
+  for (int w = 1; w < streams; ++w) Mr = fmaxf(Mr, s_max[w][row]);
+  // attention sink: one more term in the softmax denominator, exp(sink - M), with no value attached
+  if (a.sinks && row < rows_live) tot += __expf(a.sinks[h * Ge + row0 + row] - (Mr == -INFINITY ? 0.f : Mr));
+  const float inv = tot > 0.f ? 1.f / tot : 0.f;
+  __bf16* outp = (__bf16*)a.output + (int64_t)b * a.stride_out_s + (int64_t)(h * Ge + row0 + row) * a.stride_out_h +
+                 chunk * kWideDims + d;
+  *outp = row < rows_live ? (__bf16)(o * inv) : (__bf16)0.f;
+}
+
 }  // namespace
 
 #endif  // PA_REDUCE_KERNEL_H_
