@@ -1,10 +1,12 @@
 #!/usr/bin/env python3
 """Benchmark of the paged-attention decode hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]            the headline (c2) plus the other configurations
+    python bench.py [--gpus 1] [--steps K] [--warmup W]            the headline (c2) plus c2 and c4 at the reference's
+                                                                     256-token partitions, c3, c4 and c5 in `configs`
     python bench.py --workload c1|c2|c3|c4|c5 [--partition-size N]   one configuration
     python bench.py --workload ref:B,Hq,Hkv,bs,qlen[,transv][,ctx=N]  one row of the reference harness's sweep
     python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1]
+                               [,lens=c5[,qlens=c5|N][,pick=one|rest]]   c5's draw of context lengths (and of new tokens per sequence)
     python bench.py --workload probe_gather                          read-only probe of c2's page-gather pattern
     python bench.py --workload probe_issue                           issue cost of the decode step's instructions
     python bench.py --workload kv_write | kv_quantize                the KV-cache write kernels, the step before the path
@@ -118,13 +120,33 @@ def _make_custom_workload(spec, device, seed):
     q, ctx, bs = int(kv.get("q", 1)), int(kv.get("ctx", 4096)), int(kv.get("bs", 16))
     scale, kvd, qd = kv.get("scale", "tensor"), kv.get("kv", "fp8"), kv.get("qdtype", "bf16")
     transv = kv.get("transv", "0") == "1"
-    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv"}
+    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv", "lens", "qlens", "pick"}
     if unknown:
         raise ValueError(f"custom: unknown keys {sorted(unknown)}")
+    ctx_lens, q_lens, tag = torch.full((b,), ctx, dtype=torch.int32), None, f"ctx{ctx}"
+    if kv.get("lens") == "c5":
+        # the ragged configuration's own draw of context lengths (and of new tokens per sequence: qlens=c5), for
+        # experiments that vary one thing about it; qlens=N gives every sequence N new tokens in buffers padded to q
+        gen = W._gen("cpu", 5, 9)
+        ctx_lens = W._lognormal_ctx(b, 2048, 1.0, 16, 65536, gen)
+        drawn = torch.randint(1, 5, (b,), generator=gen, dtype=torch.int32)
+        tag = "c5lens"
+        if "qlens" in kv:
+            q_lens = drawn if kv["qlens"] == "c5" else torch.full((b,), int(kv["qlens"]), dtype=torch.int32)
+            q_lens = torch.clamp(q_lens, max=q)
+            ctx_lens = torch.maximum(ctx_lens, q_lens)
+            tag += f"_qlens{kv['qlens']}"
+        if "pick" in kv:  # pick=one: only the sequences that drew one new token; pick=rest: the others
+            keep = (drawn == 1) if kv["pick"] == "one" else (drawn != 1)
+            ctx_lens, b = ctx_lens[keep], int(keep.sum())
+            q_lens = None if q_lens is None else q_lens[keep]
+            tag += f"_pick{kv['pick']}"
+    elif "lens" in kv or "qlens" in kv:
+        raise ValueError("custom: lens=c5 is the only length distribution on offer; qlens needs it")
     wl = W.make_decode_workload(
-        name=f"custom_b{b}_h{hq}x{hkv}_bs{bs}_q{q}_ctx{ctx}_{kvd}_{scale}_{qd}q{'_transv' if transv else ''}", seed=seed,
+        name=f"custom_b{b}_h{hq}x{hkv}_bs{bs}_q{q}_{tag}_{kvd}_{scale}_{qd}q{'_transv' if transv else ''}", seed=seed,
         batch=b, num_q_heads=hq, num_kv_heads=hkv, block_size=bs,
-        context_lens=torch.full((b,), ctx, dtype=torch.int32), q_len=q, kv_dtype=kvd,
+        context_lens=ctx_lens, q_len=q, q_lens=q_lens, kv_dtype=kvd,
         scale_mode="none" if kvd == "bf16" else scale, device=device, transposed_v=transv)
     if qd == "fp8":
         q8, q8s = L.pertoken_quant(wl.query.float())
@@ -188,10 +210,12 @@ class _Config:
         self.plans = []
         for wl in self.wls:
             out = torch.empty(wl.query.shape, dtype=torch.bfloat16, device=dev)
+            # the two context-length statistics a serving engine has on the host: the longest and the sum
             self.plans.append(T.plan_decode(
                 out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
                 wl.q_len, wl.max_context_len, torch.bfloat16, wl.meta.get("query_scale"), wl.key_scale, wl.value_scale,
-                partition_size=partition_size or None, query_lens=wl.q_lens))
+                partition_size=partition_size or None, query_lens=wl.q_lens,
+                total_context_tokens=int(wl.context_lens.to(torch.int64).sum())))
         self.wl0 = self.wls[0]
         self.kv_bytes = self.wl0.kv_bytes()
         self.partition_size = int(self.plans[0].args.partition_size)
@@ -223,6 +247,7 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
     # event pair brackets `steps` back-to-back launches, which is what a kernel trace's average sees; otherwise other
     # kernels run in between and every launch gets an event pair of its own (which also brackets its dispatch).
     solo = plans[0].args.max_num_partitions == 1
+    r_us_avg = None
     if solo:
         k_launches = max(steps, 100)  # (a short run's 20 launches would mostly measure the first one's ramp)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -236,7 +261,7 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
         k_us_avg = e0.elapsed_time(e1) * 1e3 / k_launches
         k_timing = f"one event pair around {k_launches} back-to-back launches"
     else:
-        kevs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        kevs = [tuple(torch.cuda.Event(enable_timing=True) for _ in range(3)) for _ in range(steps)]
         for i in range(steps):
             p = plans[i % n]
             kevs[i][0].record(stream)
@@ -245,9 +270,13 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
             if rc:
                 _cabi.check(rc, "pa_decode_partition")
             lib.pa_decode_reduce(C.byref(p.args), sh)
+            kevs[i][2].record(stream)
         torch.cuda.synchronize()
-        k_us = [e0.elapsed_time(e1) * 1e3 for e0, e1 in kevs]
+        k_us = [e0.elapsed_time(e1) * 1e3 for e0, e1, _ in kevs]
         k_us_avg = sum(k_us) / len(k_us)
+        # (stage 2 over every sequence, as pa_decode_reduce runs it alone; inside pa_decode it skips the sequences
+        # stage 1 has finished)
+        r_us_avg = sum(e1.elapsed_time(e2) * 1e3 for _, e1, e2 in kevs) / len(kevs)
         k_timing = "an event pair around every launch (planning kernel included when the launch uses one)"
 
     # ---- the whole op
@@ -267,7 +296,7 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
     torch.cuda.synchronize()
     call_us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
     return {"us_median": call_us[len(call_us) // 2], "us_mean": sum(call_us) / len(call_us), "wall_ms": wall_ms,
-            "kernel_us_avg": k_us_avg, "kernel_timing": k_timing}
+            "kernel_us_avg": k_us_avg, "kernel_timing": k_timing, "reduce_us_avg": r_us_avg}
 
 
 def _sample_power(lib, cfg, stream, seconds):
@@ -345,6 +374,8 @@ def _config_line(cfg, t):
         "workload": cfg.wl0.name, "partition_size": cfg.partition_size, "us_per_call": round(t["us_median"], 2),
         "kv_GBps": round(cfg.kv_bytes / (t["us_median"] * 1e-6) / 1e9, 1), "kernel": cfg.kernel, "launch": cfg.launch,
         "kernel_us_avg": round(t["kernel_us_avg"], 2), "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "reduce_us_avg": None if t["reduce_us_avg"] is None else round(t["reduce_us_avg"], 2),
+        "partitions_per_sequence": int(cfg.plans[0].args.max_num_partitions),
         "algorithmic_bytes_per_launch": cfg.kv_bytes,
         "reference_formula_TBps": round(_reference_bandwidth_tbps(cfg.wl0, t["us_median"]), 3),
     }
@@ -473,6 +504,12 @@ def _bench_decode(a) -> int:
         for name in ("c3", "c4", "c5"):
             other = _Config(name, dev, 1)  # each of them streams far more than the last-level cache holds
             lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 30), 5, a.settle)))
+            if name == "c4":
+                # ... and at the configuration's literal partition size: 512 partitions per sequence, the merge of
+                # which is what the configuration is there to stress
+                c4_256 = _Config("c4", dev, 1, 256, shared_from=other)
+                lines.append(_config_line(c4_256, _time_config(lib, c4_256, stream, min(a.steps, 30), 5, a.settle)))
+                del c4_256
             del other
             torch.cuda.empty_cache()
         result["configs"] = lines

@@ -154,11 +154,19 @@ int64_t pa_decode_workspace_bytes(int32_t num_seqs, int32_t max_num_partitions);
 /*
  * Launch-time tuning layer; replaces the constants and the 15 lines of kernel selection in
  * pa_decode_triton_gluon_fp8.py:24,1492-1509,1563-1564.  Given the batch shape and the longest
- * context, returns the partition size (a multiple of 256) the partition kernel should use.
+ * context (the caller's max_sequence_length), returns the partition size (a multiple of 256) the partition kernel should use.
  * Pure host arithmetic; num_cus <= 0 means "ask the current device".
  */
 int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int32_t rows_per_group,
                                     int32_t max_context_len, int32_t block_size, int32_t num_cus);
+/*
+ * The same with one more statistic of the context lengths, which every serving engine has on the host: their sum
+ * (0 or less: unknown, every sequence is taken to be as long as the longest).  A batch whose tokens sit in a few
+ * long sequences gets the smaller partitions that fill the GPU from those few.
+ */
+int pa_decode_select_partition_size_stats(int32_t num_seqs, int32_t num_kv_heads, int32_t rows_per_group,
+                                          int32_t max_context_len, int64_t total_context_tokens, int32_t block_size,
+                                          int32_t num_cus);
 
 /*
  * Stage 1: for every (sequence, kv head, partition) gathers the partition's KV pages through

@@ -101,6 +101,23 @@ def test_partition_size_choices():
         f(0, 8, 8, 4096, 16, 256)
 
 
+def test_partition_size_from_the_longest_context_and_the_total():
+    """The tuning layer's second statistic: the sum of the context lengths.  A batch counts as total / longest
+    sequences of the longest length, so a batch whose tokens sit in one or two long sequences gets the small
+    partitions of a small batch (measured on the GPU: 8 sequences, one of 65536 tokens and seven of 1024, 32 rows per
+    kv head: 132.6 us at 5632 against 51.5 us at 1536); an even batch, or no total, changes nothing."""
+    f = T.select_partition_size
+    # (num_seqs, kv heads, rows per group, longest context, block size, CUs, total tokens)
+    assert f(8, 8, 32, 65536, 16, 256) == 5632 and f(8, 8, 32, 65536, 16, 256, 65536 + 7 * 1024) == 1536
+    assert f(8, 8, 8, 65536, 16, 256) == 8192 and f(8, 8, 8, 65536, 16, 256, 65536 + 7 * 1024) == 2048
+    assert f(32, 8, 8, 32768, 16, 256, 2 * 32768 + 30 * 512) == 2048
+    assert f(64, 8, 8, 4096, 16, 256, 64 * 4096) == f(64, 8, 8, 4096, 16, 256) == 4096     # c2: even
+    assert f(256, 8, 64, 28856, 16, 256, 896879) == f(256, 8, 64, 28856, 16, 256) == 7424  # c5: 8192-token cap either way
+    assert f(8, 8, 32, 65536, 16, 256, 8 * 65536) == f(8, 8, 32, 65536, 16, 256)           # total = batch x longest
+    assert f(8, 8, 32, 65536, 16, 256, 10 ** 12) == f(8, 8, 32, 65536, 16, 256)            # never more than the batch
+    assert f(8, 8, 32, 65536, 16, 256, 5) == f(1, 8, 32, 65536, 16, 256)                   # never less than one sequence
+
+
 def _cpu_args(**over):
     wl = W.make_decode_workload(name="v", seed=1, batch=2, num_q_heads=8, num_kv_heads=2,
                                 context_lens=torch.tensor([40, 300], dtype=torch.int32))

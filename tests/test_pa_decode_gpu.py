@@ -664,6 +664,10 @@ def test_scaled_down_benchmark_configs(cuda, name, batch, ctx_scale):
     print(f"config={wl.name} ctx={wl.context_lens.tolist()}", flush=True)
     out, res = _run(wl, cuda, partition_size=None)
     torch.testing.assert_close(out.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+    # the tuning layer with the second statistic, the sum of the context lengths (a host value)
+    out2, res2 = _run(wl, cuda, partition_size=None, total_context_tokens=int(wl.context_lens.sum()))
+    torch.testing.assert_close(out2.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+    assert res2["partition_size"] <= res["partition_size"]  # fewer tokens than batch x longest: never coarser
 
 
 def _random_case(seed):

@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "pa_decode_last_hip_error",
     "pa_decode_workspace_bytes",
     "pa_decode_select_partition_size",
+    "pa_decode_select_partition_size_stats",
     "pa_decode_partition",
     "pa_decode_reduce",
     "pa_decode",
@@ -101,6 +102,8 @@ def load_library(path: str = None) -> C.CDLL:
         lib.pa_decode_workspace_bytes.argtypes = [C.c_int32, C.c_int32]
         lib.pa_decode_select_partition_size.restype = C.c_int
         lib.pa_decode_select_partition_size.argtypes = [C.c_int32] * 6
+        lib.pa_decode_select_partition_size_stats.restype = C.c_int
+        lib.pa_decode_select_partition_size_stats.argtypes = [C.c_int32] * 4 + [C.c_int64, C.c_int32, C.c_int32]
         for name in ("pa_decode_partition", "pa_decode_reduce", "pa_decode", "pa_decode_noalloc"):
             fn = getattr(lib, name)
             fn.restype = C.c_int

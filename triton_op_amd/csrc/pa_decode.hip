@@ -361,9 +361,11 @@ int launch_reduce(const PaDecodeArgs* a, void* hip_stream, bool skip_single) {
   if (blocks <= 2LL * device_num_cus() && a->max_num_partitions >= 64 && (a->stride_tmp_g * 2) % 16 == 0 &&
       (a->stride_tmp_p * 2) % 16 == 0 && (a->stride_tmp_h * 2) % 16 == 0 && (a->stride_tmp_s * 2) % 16 == 0 &&
       (reinterpret_cast<uintptr_t>(a->tmp_output) & 15) == 0)
-    return skip_single
-               ? pa_launch(pa_reduce_wide_kernel<true>, dim3((unsigned)blocks * kWideDimSplit), dim3(64 * kWideWaves), 0, stream, *a)
-               : pa_launch(pa_reduce_wide_kernel<false>, dim3((unsigned)blocks * kWideDimSplit), dim3(64 * kWideWaves), 0, stream, *a);
+  {
+    const dim3 wide((unsigned)((blocks + 7) / 8 * 8 * kWideDimSplit));  // (whole groups of eight units: see the kernel)
+    return skip_single ? pa_launch(pa_reduce_wide_kernel<true>, wide, dim3(64 * kWideWaves), 0, stream, *a)
+                       : pa_launch(pa_reduce_wide_kernel<false>, wide, dim3(64 * kWideWaves), 0, stream, *a);
+  }
   if (skip_single)
     return big ? pa_launch(pa_reduce_kernel<true, 4>, grid, dim3(256), 0, stream, *a)
                : pa_launch(pa_reduce_kernel<true, 1>, grid, dim3(1024), 0, stream, *a);
@@ -411,9 +413,26 @@ const char* pa_decode_error_string(int code) {
 
 int pa_decode_select_partition_size(int32_t num_seqs, int32_t num_kv_heads, int32_t rows_per_group,
                                     int32_t max_context_len, int32_t block_size, int32_t num_cus) {
+  return pa_decode_select_partition_size_stats(num_seqs, num_kv_heads, rows_per_group, max_context_len, 0, block_size,
+                                               num_cus);
+}
+
+int pa_decode_select_partition_size_stats(int32_t num_seqs_given, int32_t num_kv_heads, int32_t rows_per_group,
+                                          int32_t max_context_len, int64_t total_context_tokens, int32_t block_size,
+                                          int32_t num_cus) {
   (void)block_size;
-  if (num_seqs <= 0 || num_kv_heads <= 0 || max_context_len <= 0 || rows_per_group <= 0) return PA_ERR_BAD_SHAPE;
+  if (num_seqs_given <= 0 || num_kv_heads <= 0 || max_context_len <= 0 || rows_per_group <= 0) return PA_ERR_BAD_SHAPE;
   if (num_cus <= 0) num_cus = device_num_cus();
+  // The longest context sets how long the longest sequence's workgroups run; how many workgroups there are to fill
+  // the GPU with is a matter of the batch's TOTAL length.  A batch of uneven lengths counts as total / longest
+  // sequences of the longest length (8 sequences of which one holds nine tenths of the tokens are little more than
+  // one sequence, and want the many small partitions that a batch of one wants).  Unknown total: every sequence
+  // is taken to be as long as the longest.
+  int num_seqs = num_seqs_given;
+  if (total_context_tokens > 0) {
+    const long long eff = (total_context_tokens + max_context_len - 1) / max_context_len;
+    num_seqs = (int)(eff < 1 ? 1 : (eff > num_seqs_given ? num_seqs_given : eff));
+  }
   const int total_tiles = (rows_per_group + 15) / 16;
   if (use_shared_stream(PA_DTYPE_FP8_E4M3FN, rows_per_group)) {
     // All row tiles of a kv head in one workgroup that walks its partition alone: three workgroups fit a CU, and

@@ -224,9 +224,15 @@ __global__ __launch_bounds__(64 * kWideWaves) void pa_reduce_wide_kernel(const P
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int Ge = a.q_len * a.group_size;
   const int RT = (Ge + 15) / 16;
+  // Workgroup ids go round the GPU's eight XCDs, each with an L2 of its own; the workgroups of one unit share the
+  // 128-byte lines of its rows, so they get ids that land on ONE XCD: id = xcd + 8 * (chunk + kWideDimSplit * (unit / 8)),
+  // unit % 8 == xcd (the grid is padded to whole groups of eight units).
   long long wid = blockIdx.x;
+  const int xcd = (int)(wid % 8);
+  wid /= 8;
   const int chunk = (int)(wid % kWideDimSplit);
-  wid /= kWideDimSplit;
+  wid = (wid / kWideDimSplit) * 8 + xcd;
+  if (wid >= (long long)RT * a.num_kv_heads * a.num_seqs) return;
   const int rt = (int)(wid % RT);
   const int h = (int)((wid / RT) % a.num_kv_heads);
   const int b = (int)(wid / ((long long)RT * a.num_kv_heads));

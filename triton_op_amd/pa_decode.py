@@ -16,6 +16,9 @@ pa_decode_triton.py:523-685.  Differences, all additive:
   reference kernels index, :323-327) or one per query head ([num_kv_heads * group]);
 * `partition_size` may be any multiple of 256 (the reference's constant); by default the tuning
   layer picks it from the batch shape and the longest context;
+* `total_context_tokens` (a host integer: the sum of `sequence_lengths`, which a serving engine has at hand) is the
+  second context-length statistic the tuning layer uses beside `max_sequence_length`; nothing is read back from the
+  device for it;
 * `query_lens` gives a per-sequence number of new tokens (ragged MTP batches);
 * `sinks` gives an attention-sink logit per query row ([num_kv_heads * query_group_size], as the reference's
   Gluon reduce kernel indexes it, pa_decode_triton_gluon_fp8.py:1118-1123): exp(sink - max) joins the softmax
@@ -57,14 +60,15 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 @functools.lru_cache(maxsize=4096)
 def select_partition_size(num_seqs: int, num_kv_heads: int, rows_per_group: int, max_context_len: int,
-                          block_size: int, num_cus: int = 0) -> int:
-    """The tuning layer's choice of tokens per partition (a multiple of 256).  A pure function of its
-    arguments (and of the GPU's CU count when num_cus is 0), hence cached."""
+                          block_size: int, num_cus: int = 0, total_context_tokens: int = 0) -> int:
+    """The tuning layer's choice of tokens per partition (a multiple of 256) from the batch shape and the context
+    lengths' statistics: the longest and, when the caller knows it (a host value: nothing is read back from the
+    device), their sum.  A pure function of its arguments (and of the GPU's CU count when num_cus is 0), hence cached."""
     lib = _cabi.load_library()
-    ps = lib.pa_decode_select_partition_size(num_seqs, num_kv_heads, rows_per_group, max(1, max_context_len),
-                                             block_size, num_cus)
+    ps = lib.pa_decode_select_partition_size_stats(num_seqs, num_kv_heads, rows_per_group, max(1, max_context_len),
+                                                   int(total_context_tokens), block_size, num_cus)
     if ps < 0:
-        _cabi.check(ps, "pa_decode_select_partition_size")
+        _cabi.check(ps, "pa_decode_select_partition_size_stats")
     return ps
 
 
@@ -139,6 +143,7 @@ def plan_decode(
     workspace: Optional[torch.Tensor] = None,
     sinks: Optional[torch.Tensor] = None,
     reuse_item_list: bool = False,
+    total_context_tokens: int = 0,
 ) -> DecodePlan:
     if temp_output is not None:  # the spelling of run_gluon_fp8_kernel (test_pa_mtp.py:566-584)
         if tmp_output is not None and tmp_output is not temp_output:
@@ -289,7 +294,8 @@ def plan_decode(
             per = -(-max_seq // int(num_sequence_partitions))
             partition_size = -(-per // PARTITION_GRANULE) * PARTITION_GRANULE
         else:
-            partition_size = select_partition_size(num_seqs, num_kv_heads, ge, max_seq, block_size)
+            partition_size = select_partition_size(num_seqs, num_kv_heads, ge, max_seq, block_size, 0,
+                                                   int(total_context_tokens))
     partition_size = int(partition_size)
     if partition_size <= 0 or partition_size % PARTITION_GRANULE:
         raise ValueError(f"partition_size must be a positive multiple of {PARTITION_GRANULE}, got {partition_size}")
@@ -398,6 +404,7 @@ def paged_attention_decode(
     workspace: Optional[torch.Tensor] = None,
     sinks: Optional[torch.Tensor] = None,
     reuse_item_list: bool = False,
+    total_context_tokens: int = 0,
 ) -> Dict[str, object]:
     """Split-KV paged-attention decode; writes `output` in place on torch's current stream and
     returns the partition buffers under the reference's keys."""
@@ -406,7 +413,7 @@ def paged_attention_decode(
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
         num_sequence_partitions, alibi_slopes, max_logits, exp_sums, tmp_output, temp_output=temp_output,
         partition_size=partition_size, query_lens=query_lens, workspace=workspace,
-        sinks=sinks, reuse_item_list=reuse_item_list)
+        sinks=sinks, reuse_item_list=reuse_item_list, total_context_tokens=total_context_tokens)
     plan.run()
     return {
         "temporary_output": plan.tmp_output,
