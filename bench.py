@@ -50,6 +50,15 @@ HBM_TRAFFIC = {
     ("c2_fp8_b64_ctx4k", 256): {
         "bytes": 556_600_000, "launch": "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 4 partitions per workgroup",
         "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
+    ("c3_fp8_mtp2_bs1024", 8192): {
+        "bytes": 4_437_300_000, "launch": "pa_partition_kernel<fp8, strided, 4 waves> x 4096, sorted items",
+        "profile": "profiles/pa_partition_kernel_c3_c4_hbm_traffic.md"},
+    ("c4_fp8_ctx128k", 8192): {
+        "bytes": 1_077_200_000, "launch": "pa_partition_kernel<fp8, bs16, 4 waves> x 512",
+        "profile": "profiles/pa_partition_kernel_c3_c4_hbm_traffic.md"},
+    ("c4_fp8_ctx128k", 256): {
+        "bytes": 1_110_800_000, "launch": "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 8 partitions per workgroup",
+        "profile": "profiles/pa_partition_kernel_c3_c4_hbm_traffic.md"},
     ("c5_ragged_mix", 7424): {
         "bytes": 2_050_500_000,
         "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items",
@@ -377,6 +386,7 @@ def _config_line(cfg, t):
         "reduce_us_avg": None if t["reduce_us_avg"] is None else round(t["reduce_us_avg"], 2),
         "partitions_per_sequence": int(cfg.plans[0].args.max_num_partitions),
         "algorithmic_bytes_per_launch": cfg.kv_bytes,
+        "traffic": _traffic(cfg)[0],  # HBM bytes per launch of the partition kernel by FETCH_SIZE + WRITE_SIZE (profiles/)
         "reference_formula_TBps": round(_reference_bandwidth_tbps(cfg.wl0, t["us_median"]), 3),
     }
 

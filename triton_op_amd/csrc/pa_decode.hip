@@ -241,9 +241,15 @@ int launch_plan(const PaDecodeArgs& a, hipStream_t stream) {
 template <int NT, int KVT, bool PT, bool BS16, int W>
 int launch_partition_w(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
   constexpr int OCC = NT == 1 ? 2 : 1;
-  if (c.queue)
-    return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>, dim3((unsigned)c.blocks), dim3(64 * W), 0, stream, k);
-  return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>, dim3((unsigned)c.blocks), dim3(64 * W), 0, stream, k);
+  const dim3 grid((unsigned)c.blocks), block(64 * W);
+  if constexpr (NT == 2) {
+    // more rows per kv head than one workgroup's two tiles: another workgroup reads the same pages (see REREAD)
+    if (k.q_len * k.group_size > 32)
+      return c.queue ? pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true, true>, grid, block, 0, stream, k)
+                     : pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false, true>, grid, block, 0, stream, k);
+  }
+  if (c.queue) return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>, grid, block, 0, stream, k);
+  return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>, grid, block, 0, stream, k);
 }
 
 template <int NT, int KVT, bool PT, bool BS16>

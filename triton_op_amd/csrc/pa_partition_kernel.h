@@ -55,7 +55,10 @@ struct StepData {
 // of a tile share one address register pair and differ by immediate offsets.
 constexpr int kQueueMaxSeqs = 2048;  // sequences the item table of the queued launch can hold
 
-template <int NT, int KVT, bool PER_TOKEN, bool BS16, int WAVES, int OCC, bool QUEUE>
+// REREAD: the kv head has more row tiles than a workgroup takes (a bf16 cache with more than 32 query rows), so a
+// second workgroup streams the same pages at about the same time: the cache is then read with ordinary loads (the
+// lines had better still be in L2 when the other workgroup asks; non-temporal loads mark them for early eviction).
+template <int NT, int KVT, bool PER_TOKEN, bool BS16, int WAVES, int OCC, bool QUEUE, bool REREAD = false>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_kernel(const PaDecodeArgs a) {
   constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
@@ -283,12 +286,18 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     }
     return pg;
   };
+  constexpr bool read_once = !REREAD;  // (a choice made per load at run time costs a tenth of the kernel's rate)
   auto issue_k = [&](SD& sd, const Pages& pg) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const char* tb = kbase + (int64_t)pg.p[j] * k_block_bytes + (int64_t)pg.off[j] * 16;
+      if constexpr (read_once) {
 #pragma unroll
-      for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16_stream(tb + k_lane_off[ld]);
+        for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16_stream(tb + k_lane_off[ld]);
+      } else {
+#pragma unroll
+        for (int ld = 0; ld < SD::NKL; ++ld) sd.k[j][ld] = load16(tb + k_lane_off[ld]);
+      }
       if constexpr (PER_TOKEN) {
         const int64_t so = (int64_t)pg.p[j] * a.stride_kvscale_b + pg.off[j] + 4 * kg;
         sd.ks[j] = *reinterpret_cast<const f32x4*>(ksbase + so);
@@ -303,7 +312,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     // Non-temporal where one load covers whole 128-byte lines.  With plain V and pages of more than 64 tokens
     // a 64-token step takes half a line of every head dim's row and the next step the other half: those lines
     // must stay in L2 in between (streaming them costs 13 % on 1024-token pages).
-    if (BS16 || v_whole_lines) {
+    if ((BS16 || v_whole_lines) && read_once) {
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
 #pragma unroll
