@@ -8,6 +8,9 @@
     python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1]
                                [,lens=c5[,qlens=c5|N][,pick=one|rest]]   c5's draw of context lengths (and of new tokens per sequence)
     python bench.py --workload probe_gather                          read-only probe of c2's page-gather pattern
+    python bench.py --workload probe_gather:c5                       ... of another workload's (plain order, four-wave workgroups)
+    python bench.py --workload probe_stream42:c5                     the pages read by workgroups whose waves share each step
+                                                                     (depth 4 steps in registers, 2 workgroups per CU)
     python bench.py --workload probe_issue                           issue cost of the decode step's instructions
     python bench.py --workload kv_write | kv_quantize                the KV-cache write kernels, the step before the path
 
@@ -549,6 +552,8 @@ def _load_probe_library():
     lib = C.CDLL(path)
     lib.pa_probe_gather.restype = C.c_int
     lib.pa_probe_gather.argtypes = [C.POINTER(_cabi.PaDecodeArgs), C.c_void_p, C.c_void_p]
+    lib.pa_probe_stream.restype = C.c_int
+    lib.pa_probe_stream.argtypes = [C.POINTER(_cabi.PaDecodeArgs), C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.pa_probe_issue.restype = C.c_int
     lib.pa_probe_issue.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     return lib
@@ -570,13 +575,21 @@ def _bench_probe_gather(a) -> int:
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream(dev)
     sh = C.c_void_p(stream.cuda_stream)
-    cfg = _Config("c2", dev, a.pools, a.partition_size, a.batch or None)
+    of = a.workload.partition(":")[2] or "c2"  # probe_gather:c5, probe_gather:custom:... = that workload's pages
+    cfg = _Config(of, dev, a.pools, a.partition_size, a.batch or None)
     sink = torch.zeros(64, dtype=torch.int32, device=dev)
 
+    # probe_gather | probe_stream42 (depth 4, 2 workgroups per CU) | probe_stream42v1 (+ variant: 1 no barrier, 2 no scales)
+    shape, _, variant = a.workload.partition(":")[0].partition("v")
+
     def call(i):
-        rc = lib.pa_probe_gather(C.byref(cfg.plans[i % len(cfg.plans)].args), C.c_void_p(sink.data_ptr()), sh)
+        args = C.byref(cfg.plans[i % len(cfg.plans)].args)
+        if shape == "probe_gather":
+            rc = lib.pa_probe_gather(args, C.c_void_p(sink.data_ptr()), sh)
+        else:
+            rc = lib.pa_probe_stream(args, int(shape[-2]), int(shape[-1]), int(variant or 0), C.c_void_p(sink.data_ptr()), sh)
         if rc:
-            _cabi.check(rc, "pa_probe_gather")
+            _cabi.check(rc, shape)
 
     for i in range(a.settle):
         call(i)
@@ -590,12 +603,12 @@ def _bench_probe_gather(a) -> int:
     us = e0.elapsed_time(e1) * 1e3 / a.steps
     gbps = cfg.kv_bytes / (us * 1e-6) / 1e9
     print(json.dumps({
-        "metric": "read-only gather probe of c2's page pattern (no arithmetic)", "value": round(gbps, 1), "unit": "GB/s",
+        "metric": "read-only gather probe of %s's page pattern (no arithmetic)" % of, "value": round(gbps, 1), "unit": "GB/s",
         "us_per_call": round(us, 2), "n_gpus": 1, "steps": a.steps, "warmup": a.settle, "ms_per_step": round(us / 1e3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "probe_gather_" + cfg.wl0.name, "bytes_per_call": cfg.kv_bytes,
                    "kv_pools_rotated": len(cfg.plans)},
-        "roofline": {"bound": "hbm", "kernel": "pa_gather_probe_kernel", "achieved": round(gbps, 1),
+        "roofline": {"bound": "hbm", "kernel": "pa_gather_probe_kernel" if shape == "probe_gather" else "pa_stream_probe_kernel", "achieved": round(gbps, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None},
     }, ensure_ascii=False))
     return 0
@@ -776,7 +789,7 @@ def main() -> int:
         return 2
     if a.workload in ("kv_write", "kv_quantize"):
         return _bench_kv_cache(a)
-    if a.workload == "probe_gather":
+    if a.workload.partition(":")[0] == "probe_gather" or a.workload.startswith("probe_stream"):
         return _bench_probe_gather(a)
     if a.workload == "probe_issue":
         return _bench_probe_issue(a)

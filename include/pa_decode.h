@@ -208,8 +208,8 @@ int pa_decode(const PaDecodeArgs* args, void* hip_stream);
  *
  * Environment: none of the library's behaviour depends on environment variables unless the process was started
  * with PA_DECODE_DEBUG=1, which enables the tuning switches PA_DECODE_WAVES, PA_DECODE_ROW_TILES, PA_DECODE_SPAN,
- * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED, PA_DECODE_LDS_PAD and PA_DECODE_P_RESIDUAL (read once, at the
- * first launch).
+ * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED, PA_DECODE_LDS_PAD, PA_DECODE_P_RESIDUAL and PA_DECODE_XCD (read
+ * once, at the first launch).
  */
 int pa_decode_launch_info(const PaDecodeArgs* args, char* text, int32_t text_bytes);
 

@@ -24,6 +24,16 @@ extern "C" {
 int pa_probe_gather(const PaDecodeArgs* args, int32_t* sink, void* hip_stream);
 
 /*
+ * The same pages read by workgroups whose four waves share every 64-token step: wave w loads K of the step's tile
+ * w, head dims 32 w .. 32 w + 31 of V and the tile's per-token scales (when the arguments have them), `depth` (2, 4,
+ * 6 or 8) steps ahead in registers, with one workgroup barrier per step; `workgroups_per_cu` 2, 3 or 4 (depth 4
+ * or 6 for 4).  variant: bit 0 = no barrier, bit 1 = the per-token scales are not read (what each of the two costs).
+ * Same restrictions and sink as pa_probe_gather.
+ */
+int pa_probe_stream(const PaDecodeArgs* args, int32_t depth, int32_t workgroups_per_cu, int32_t variant, int32_t* sink,
+                    void* hip_stream);
+
+/*
  * The issue cost of the instructions the decode step is made of.  Launches `workgroups` workgroups of four waves
  * (one per SIMD; 256 x n workgroups put n waves on every SIMD of a 256-CU GPU) that each run `iterations` x 128
  * instructions of one kind: mode 0 v_fma_f32 (the full-rate yardstick), 3 v_exp_f32, 4 v_cvt_pk_fp8_f32,

@@ -35,6 +35,39 @@ int pa_probe_gather(const PaDecodeArgs* a, int32_t* sink, void* hip_stream) {
                 reinterpret_cast<int*>(sink));
 }
 
+int pa_probe_stream(const PaDecodeArgs* a, int32_t depth, int32_t workgroups_per_cu, int32_t variant, int32_t* sink,
+                    void* hip_stream) {
+  if (!a || !sink) return PA_ERR_NULL_POINTER;
+  if (a->struct_size != sizeof(PaDecodeArgs)) return PA_ERR_BAD_STRUCT;
+  if (!a->key_cache || !a->value_cache || !a->context_lens || !a->block_tables) return PA_ERR_NULL_POINTER;
+  if (a->num_seqs <= 0 || a->num_kv_heads <= 0 || a->max_num_partitions <= 0 || a->partition_size <= 0 ||
+      a->partition_size % 256)
+    return PA_ERR_BAD_SHAPE;
+  if (a->kv_dtype != PA_DTYPE_FP8_E4M3FN || a->block_size != 16 || a->stride_k_c != 256 || a->stride_v_2 != 16 ||
+      a->v_transposed || a->head_size != kHeadSize)
+    return PA_ERR_UNSUPPORTED;
+  if (a->kv_quant_mode == PA_QUANT_PER_TOKEN && (!a->key_scale || !a->value_scale)) return PA_ERR_NULL_POINTER;
+  const long long blocks = (long long)a->num_seqs * a->num_kv_heads * a->max_num_partitions;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  const dim3 grid((unsigned)blocks), block(256);
+  int* s = reinterpret_cast<int*>(sink);
+  const int v = variant;
+  switch (depth * 10 + workgroups_per_cu) {
+    case 22: return launch(pa_stream_probe_kernel<2, 2>, grid, block, stream, *a, s, v);
+    case 42: return launch(pa_stream_probe_kernel<4, 2>, grid, block, stream, *a, s, v);
+    case 62: return launch(pa_stream_probe_kernel<6, 2>, grid, block, stream, *a, s, v);
+    case 23: return launch(pa_stream_probe_kernel<2, 3>, grid, block, stream, *a, s, v);
+    case 43: return launch(pa_stream_probe_kernel<4, 3>, grid, block, stream, *a, s, v);
+    case 63: return launch(pa_stream_probe_kernel<6, 3>, grid, block, stream, *a, s, v);
+    case 44: return launch(pa_stream_probe_kernel<4, 4>, grid, block, stream, *a, s, v);
+    case 64: return launch(pa_stream_probe_kernel<6, 4>, grid, block, stream, *a, s, v);
+    case 82: return launch(pa_stream_probe_kernel<8, 2>, grid, block, stream, *a, s, v);
+    case 83: return launch(pa_stream_probe_kernel<8, 3>, grid, block, stream, *a, s, v);
+    default: return PA_ERR_UNSUPPORTED;
+  }
+}
+
 int pa_probe_issue(int32_t mode, int32_t iterations, int32_t workgroups, int32_t* sink, void* hip_stream) {
   if (!sink) return PA_ERR_NULL_POINTER;
   if (iterations <= 0 || workgroups <= 0) return PA_ERR_BAD_SHAPE;

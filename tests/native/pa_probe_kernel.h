@@ -84,6 +84,101 @@ void pa_gather_probe_kernel(const PaDecodeArgs a, int* sink) {
   if (__builtin_amdgcn_ballot_w64(fold != 0x9e3779b9u) == 0) sink[lane] = (int)fold;
 }
 
+// pa_stream_probe_kernel: the same pages read the way a workgroup would read them whose four waves work on the SAME
+// 64-token step: wave w loads K of the step's tile w (2 KiB), the 32 head dims 32 w .. 32 w + 31 of V for all four
+// tiles (2 KiB) and, with per-token scales, the tile's 16 + 16 scales, DEPTH steps ahead of the step it folds, in
+// registers; one workgroup barrier per step stands for the exchange of the step's probabilities.  OCC workgroups per
+// CU.  What this reaches is what such a kernel could reach before its arithmetic.
+template <int DEPTH, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+void pa_stream_probe_kernel(const PaDecodeArgs a, int* sink, int variant) {
+  const bool with_barrier = !(variant & 1);  // variant bit 0: no barrier between the steps
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, kg = lane >> 4;
+  const int Hkv = a.num_kv_heads;
+  const long long wid = blockIdx.x;
+  const int h = (int)(wid % Hkv);
+  const long long item = wid / Hkv;
+  const int b = (int)(item % a.num_seqs);
+  const int part = (int)(item / a.num_seqs);
+  const int ctx = sload_i32(a.context_lens + b);
+  const int wg_start = part * a.partition_size;
+  if (wg_start >= ctx) return;
+  const int wg_end = min(wg_start + a.partition_size, ctx);
+  const int n_steps = (wg_end - wg_start + kStepTokens - 1) / kStepTokens;
+  const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h;
+  const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h;
+  const bool per_token = a.kv_quant_mode == PA_QUANT_PER_TOKEN && !(variant & 2);  // bit 1: the scales are not read
+  // (without per-token scales the load reads one word of the context lengths instead: no branch around a load)
+  const float* sc_lane = per_token ? ((lane & 16) ? a.value_scale : a.key_scale) + (int64_t)h * a.stride_kvscale_h + li
+                                   : reinterpret_cast<const float*>(a.context_lens);
+  const int64_t sc_page_stride = per_token ? a.stride_kvscale_b : 0;
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const int last_tile_tok = (wg_end - 1) & ~15;
+  const uint32_t k_off = (uint32_t)(kg * 256 + li * 16);
+  const uint32_t v_off = (uint32_t)((32 * wave + li) * 16);
+  struct Step {
+    u32x4 k[2];
+    u32x4 v[2];
+    float sc;
+  };
+  auto issue = [&](Step& st, int tok0) {
+    int page[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int t = tok0 + 16 * j;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      page[j] = sload_i32(bt + (t >> 4));
+    }
+    int tw = tok0 + 16 * wave;
+    tw = tw > last_tile_tok ? last_tile_tok : tw;
+    const int kp = sload_i32(bt + (tw >> 4));
+    const char* tb = kbase + (int64_t)kp * a.stride_k_b;
+    st.k[0] = load16_stream(tb + k_off);
+    st.k[1] = load16_stream(tb + k_off + 1024);
+    int vp = page[0];  // (lane-wise selects, no branches)
+    vp = kg == 1 ? page[1] : vp;
+    vp = kg == 2 ? page[2] : vp;
+    vp = kg == 3 ? page[3] : vp;
+    const char* vb = vbase + (int64_t)vp * a.stride_v_b;
+    st.v[0] = load16_stream(vb + v_off);
+    st.v[1] = load16_stream(vb + v_off + 256);
+    st.sc = __builtin_nontemporal_load(sc_lane + (int64_t)kp * sc_page_stride);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  uint32_t fold = 0;
+  auto consume = [&](const Step& st) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      fold ^= st.k[i][0] ^ st.k[i][1] ^ st.k[i][2] ^ st.k[i][3] ^ st.v[i][0] ^ st.v[i][1] ^ st.v[i][2] ^ st.v[i][3];
+    fold ^= __float_as_uint(st.sc);
+    // the step's registers are needed HERE (the compiler may not gather the folds of a round at its end)
+    asm volatile("" ::"v"(st.k[0]), "v"(st.k[1]), "v"(st.v[0]), "v"(st.v[1]), "v"(st.sc));
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // whole rounds of DEPTH steps (steps past the end re-read the last tile's lines): every path to a use has issued
+  // the same loads in the same order, so the compiler's counted waits stay partial
+  Step st[DEPTH];
+  int tok = wg_start;
+#pragma unroll
+  for (int i = 0; i < DEPTH; ++i) {
+    issue(st[i], tok);
+    tok += kStepTokens;
+  }
+  const int rounds = (n_steps + DEPTH - 1) / DEPTH;
+  for (int r = 0; r < rounds; ++r) {
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) {
+      consume(st[i]);
+      if (with_barrier) __syncthreads();
+      issue(st[i], tok);
+      tok += kStepTokens;
+    }
+  }
+  if (__builtin_amdgcn_ballot_w64(fold != 0x9e3779b9u) == 0) sink[lane] = (int)fold;
+}
+
 // pa_issue_probe_kernel: what instructions of the decode step cost the issue port of a SIMD.  Every wave runs
 // `iters` iterations of 128 instructions of one kind on eight independent registers (MODE 0: v_fma_f32, the
 // full-rate yardstick; 3: v_exp_f32; 4: v_cvt_pk_fp8_f32; 5: v_permlane32_swap), or of 16 MFMAs

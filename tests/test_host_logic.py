@@ -429,6 +429,9 @@ def test_launch_layer_choices(pa_lib):
         "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items"
     assert info(b=128, hq=64, hkv=4, q=2, ctx=4096, ps=4096) == \
         "pa_partition_shared_kernel<fp8, bs16, 2 ring slots, 4 workgroups per CU> x 512"
+    # ... whose grid is whole groups of eight (sequence, partition) items (an XCD takes every eighth, with all its heads)
+    assert info(b=3, hq=64, hkv=2, q=1, ctx=4096, ps=1024) == \
+        "pa_partition_shared_kernel<fp8, bs16, 2 ring slots, 4 workgroups per CU> x 32"
     # c1: a bf16 cache, 8 rows, few workgroups
     assert info(b=4, hq=8, hkv=1, q=1, ctx=1024, ps=1024, kv="bf16") == "pa_partition_kernel<bf16, strided, 4 waves> x 4"
     # a bf16 cache with 32 rows per kv head: two row tiles per workgroup; ragged with a workspace: queued

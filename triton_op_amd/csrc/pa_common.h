@@ -25,6 +25,8 @@ constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning k
 constexpr int kFlagSpanShift = 20;         // bits 20..27: partitions a one-wave workgroup walks in one pass (0 = 1)
 // experiment switch of pa_partition_shared_kernel: P without its FP8 residual
 constexpr int kFlagResidualNever = 0x40000;
+// pa_partition_shared_kernel: the kv heads of an item are consecutive workgroups of ONE XCD (see the kernel)
+constexpr int kFlagHeadsShareXcd = 0x80000;
 // ... at most: their partial results wait in LDS for the end of the pass, in a pool of kSpanPoolBytes per 16-row
 // tile; a tile of up to 8 real rows stages only those (half the bytes) and may walk twice as many partitions
 constexpr int kSpanMax = 4;
@@ -224,8 +226,12 @@ __device__ __forceinline__ void zero_output_rows(const PaDecodeArgs& a, int b, i
 __device__ __forceinline__ void dma_load16(const void* gptr, uint32_t lds_offset) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory", "m0");
 }
+template <bool STREAM = true>
 __device__ __forceinline__ void dma_load4(const void* gptr, uint32_t lds_offset) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory", "m0");
+  if constexpr (STREAM)
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off nt" ::"v"(gptr), "s"(lds_offset) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(lds_offset) : "memory", "m0");
 }
 // the same with the address split into a wave-uniform base and a 32-bit per-lane byte offset; STREAM = false
 // for bytes whose 128-byte lines other loads will touch again soon (those must stay in L2)

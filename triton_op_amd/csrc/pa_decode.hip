@@ -83,6 +83,7 @@ int device_num_cus() {
 //   PA_DECODE_SORTED=0|1 never / always the sorted dispatch (when the workspace has room)
 //   PA_DECODE_LDS_PAD=n  unused LDS per workgroup of the shared-stream kernel (lowers its occupancy)
 //   PA_DECODE_P_RESIDUAL=0  shared-stream kernel: P without its FP8 residual (every element rounded to e4m3)
+//   PA_DECODE_XCD=0         shared-stream kernel: the kv head fastest in the workgroup id (heads spread over the XCDs)
 // All are read once, at the first launch.
 int debug_switch(const char* name, int unset) {
   static const bool enabled = [] {
@@ -130,6 +131,7 @@ struct LaunchChoice {
   bool queue;       // a resident grid pulls live items from a counter in the workspace
   bool sorted;      // items come from the planning kernel's list in the workspace
   bool listed_reduce;  // ... and pa_decode's reduce stage walks the planning kernel's list of multi-partition sequences
+  bool heads_share_xcd;  // pa_partition_shared_kernel: an item's kv heads are consecutive workgroups of one XCD
   long long blocks; // workgroups launched
 };
 
@@ -141,6 +143,7 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
   c.bs16 = c.fp8 && a.block_size == 16 && a.stride_k_c == 256 &&
            (a.v_transposed ? a.stride_v_2 == 2048 : a.stride_v_2 == 16);
   c.shared = use_shared_stream(a.kv_dtype, ge);
+  static const bool xcd_off = debug_switch("PA_DECODE_XCD", 1) == 0;
   long long items;  // (sequence, partition) pairs times kv heads times row tiles
   c.row_tiles = 1;
   if (c.shared) {
@@ -148,7 +151,13 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     // workgroup per CU is worth more than a deeper ring (measured); with them it needs about 140
     c.waves = 4;
     c.per_cu = c.per_token ? 3 : 4;
-    items = (long long)a.num_seqs * a.num_kv_heads * a.max_num_partitions;
+    // An XCD takes every eighth (sequence, partition) item with all its kv heads (the heads' per-token scales of a
+    // page share 128-byte lines, which then meet in one L2; measured on the ragged 64-row mix: 341 -> 336 us, uniform
+    // batches 1 %); the grid is whole groups of eight items.  PA_DECODE_XCD=0: the head fastest in the workgroup id.
+    c.heads_share_xcd = !xcd_off;
+    items = (long long)a.num_seqs * a.max_num_partitions;
+    if (c.heads_share_xcd) items = (items + 7) / 8 * 8;
+    items *= a.num_kv_heads;
   } else {
     // no more waves than it takes to fill the GPU's wave slots (8 per CU): with 8 workgroups or more per CU one
     // wave each is best (no merge, more independent streams: 256 sequences x 8 kv heads x 512 tokens 57.7 ->
@@ -228,6 +237,12 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
   // sequences with more than one of them is not the list of the sequences the reduce stage has to merge)
   c.listed_reduce = c.sorted && c.span == 1 && !a.sinks &&
                     a.workspace_bytes >= full_workspace_bytes(a.num_seqs, a.max_num_partitions);
+  // pa_partition_kernel with per-token scales: the same placement of an item's heads (and row tiles) on one XCD
+  if (!c.shared && !c.queue && c.fp8 && c.per_token && !xcd_off) {
+    c.heads_share_xcd = true;
+    const long long units = (long long)a.num_kv_heads * ((ge + 16 * c.row_tiles - 1) / (16 * c.row_tiles));
+    c.blocks = (items / units + 7) / 8 * 8 * units;  // whole groups of eight (sequence, partition) items
+  }
   return c;
 }
 
@@ -260,8 +275,9 @@ int launch_partition_tile(const PaDecodeArgs& k, const LaunchChoice& c, hipStrea
 }
 
 template <bool PT, bool BS16>
-int launch_partition_shared(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t stream) {
+int launch_partition_shared(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t stream) {
   static const int pad = debug_switch("PA_DECODE_LDS_PAD", 0);  // experiment: unused LDS that lowers the occupancy
+  const PaDecodeArgs& k = a;
   if constexpr (PT)
     return pa_launch(pa_partition_shared_kernel<true, BS16, 3, 3>, dim3((unsigned)c.blocks), dim3(256), (unsigned)pad, stream, k);
   else
@@ -284,6 +300,7 @@ int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t s
     k.flags = kFlagSortedItems;
   }
   if (c.span > 1) k.flags |= c.span << kFlagSpanShift;
+  if (c.heads_share_xcd) k.flags |= kFlagHeadsShareXcd;
   // experiment (PA_DECODE_DEBUG=1): PA_DECODE_P_RESIDUAL=0 drops the FP8 residual of P in the shared-stream kernel
   // (every P rounded to e4m3, as the reference's kernel rounds it)
   static const int p_residual = debug_switch("PA_DECODE_P_RESIDUAL", 1);

@@ -172,9 +172,23 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     // The partition index varies slowest: in a ragged batch the partitions that only the longest
     // sequences reach (workgroups that exit at once for everybody else) come last.
     const long long wid = blockIdx.x;
-    h = (int)(wid % Hkv);
-    rt = (int)((wid / Hkv) % RT);
-    const long long item = wid / ((long long)Hkv * RT);
+    long long item;
+    if (PER_TOKEN && (a.flags & kFlagHeadsShareXcd)) {
+      // Workgroup ids go round the eight XCDs: an XCD takes every eighth item with all its kv heads and row tiles one
+      // after the other, so the 128-byte lines that hold the per-token scales of two neighbouring heads are
+      // fetched into one L2 once (with the head fastest in the id every head sits on another XCD)
+      const int xcd = (int)(wid & 7);
+      const long long slot = wid >> 3;
+      const int unit = (int)(slot % (Hkv * RT));
+      h = unit % Hkv;
+      rt = unit / Hkv;
+      item = (slot / (Hkv * RT)) * 8 + xcd;
+      if (!(a.flags & kFlagSortedItems) && item >= (long long)a.num_seqs * ((P + span - 1) / span)) return;
+    } else {
+      h = (int)(wid % Hkv);
+      rt = (int)((wid / Hkv) % RT);
+      item = wid / ((long long)Hkv * RT);
+    }
     if (a.flags & kFlagSortedItems) {
       // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
       if (item >= sload_i32(a.workspace + 2)) return;

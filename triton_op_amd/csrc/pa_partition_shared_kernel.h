@@ -46,8 +46,21 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int G = a.group_size;
   const int Ge = a.q_len * G;
   const long long wid = blockIdx.x;
-  const int h = (int)(wid % Hkv);
-  const long long item = wid / Hkv;
+  int h;
+  long long item;
+  if (a.flags & kFlagHeadsShareXcd) {
+    // Workgroup ids go round the eight XCDs.  With the head fastest in the id, the kv heads of an item land on
+    // eight different XCDs and each fetches the 128-byte lines that hold its own 64 bytes of per-token scales of a
+    // page AND its neighbour's; here an XCD takes every eighth item with all its heads one after the other, so the
+    // heads' scale lines (and nothing else: K and V are disjoint) meet in one L2.
+    const int xcd = (int)(wid & 7);
+    const long long slot = wid >> 3;
+    h = (int)(slot % Hkv);
+    item = (slot / Hkv) * 8 + xcd;
+  } else {
+    h = (int)(wid % Hkv);
+    item = wid / Hkv;
+  }
   int b, part;
   if (a.flags & kFlagSortedItems) {
     // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
@@ -55,6 +68,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);
     part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1);
   } else {
+    if (item >= (long long)a.num_seqs * a.max_num_partitions) return;  // (the grid is whole groups of eight items)
     b = (int)(item % a.num_seqs);
     part = (int)(item / a.num_seqs);
   }
@@ -146,8 +160,10 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     }
     if constexpr (PER_TOKEN) {
       // lanes 0-15: the K scales of the tile's 16 tokens, lanes 16-31: the V scales
+      // (ordinary loads: the other half of the line belongs to the neighbouring head, whose workgroup runs beside
+      // this one on the same XCD)
       if (lane < 32)
-        dma_load4(sc_lane + ((int64_t)page * a.stride_kvscale_b + off),
+        dma_load4<false>(sc_lane + ((int64_t)page * a.stride_kvscale_b + off),
                   st + (uint32_t)offsetof(StepLds, sc) + (uint32_t)wave * 128u);
     }
   };
