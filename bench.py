@@ -63,8 +63,9 @@ HBM_TRAFFIC = {
         "bytes": 1_110_800_000, "launch": "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 8 partitions per workgroup",
         "profile": "profiles/pa_partition_kernel_c3_c4_hbm_traffic.md"},
     ("c5_ragged_mix", 7424): {
-        "bytes": 2_050_500_000,
-        "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items",
+        "bytes": 1_991_300_000,
+        "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items, "
+                  "an item's heads on one XCD",
         "profile": "profiles/pa_partition_shared_kernel_c5_hbm_traffic.md"},
 }
 

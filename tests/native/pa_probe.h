@@ -25,10 +25,11 @@ int pa_probe_gather(const PaDecodeArgs* args, int32_t* sink, void* hip_stream);
 
 /*
  * The same pages read by workgroups whose four waves share every 64-token step: wave w loads K of the step's tile
- * w, head dims 32 w .. 32 w + 31 of V and the tile's per-token scales (when the arguments have them), `depth` (2, 4,
- * 6 or 8) steps ahead in registers, with one workgroup barrier per step; `workgroups_per_cu` 2, 3 or 4 (depth 4
- * or 6 for 4).  variant: bit 0 = no barrier, bit 1 = the per-token scales are not read (what each of the two costs).
- * Same restrictions and sink as pa_probe_gather.
+ * w, head dims 32 w .. 32 w + 31 of V and the tile's per-token scales (when the arguments have them), `depth` steps
+ * ahead in registers, with one workgroup barrier per step, `workgroups_per_cu` workgroups per CU: depth 2 or 4 with
+ * 2, 3 or 4, depth 6 with 2 (what fits the registers).  variant: bit 0 = no barrier, bit 1 = the per-token scales
+ * are not read (what each of the two costs), bit 2 = wave w reads all of V for tile w, as the waves of
+ * pa_partition_shared_kernel do.  Same restrictions and sink as pa_probe_gather.
  */
 int pa_probe_stream(const PaDecodeArgs* args, int32_t depth, int32_t workgroups_per_cu, int32_t variant, int32_t* sink,
                     void* hip_stream);

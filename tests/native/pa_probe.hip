@@ -59,11 +59,8 @@ int pa_probe_stream(const PaDecodeArgs* a, int32_t depth, int32_t workgroups_per
     case 62: return launch(pa_stream_probe_kernel<6, 2>, grid, block, stream, *a, s, v);
     case 23: return launch(pa_stream_probe_kernel<2, 3>, grid, block, stream, *a, s, v);
     case 43: return launch(pa_stream_probe_kernel<4, 3>, grid, block, stream, *a, s, v);
-    case 63: return launch(pa_stream_probe_kernel<6, 3>, grid, block, stream, *a, s, v);
+    case 24: return launch(pa_stream_probe_kernel<2, 4>, grid, block, stream, *a, s, v);
     case 44: return launch(pa_stream_probe_kernel<4, 4>, grid, block, stream, *a, s, v);
-    case 64: return launch(pa_stream_probe_kernel<6, 4>, grid, block, stream, *a, s, v);
-    case 82: return launch(pa_stream_probe_kernel<8, 2>, grid, block, stream, *a, s, v);
-    case 83: return launch(pa_stream_probe_kernel<8, 3>, grid, block, stream, *a, s, v);
     default: return PA_ERR_UNSUPPORTED;
   }
 }

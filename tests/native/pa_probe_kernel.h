@@ -88,7 +88,7 @@ void pa_gather_probe_kernel(const PaDecodeArgs a, int* sink) {
 // 64-token step: wave w loads K of the step's tile w (2 KiB), the 32 head dims 32 w .. 32 w + 31 of V for all four
 // tiles (2 KiB) and, with per-token scales, the tile's 16 + 16 scales, DEPTH steps ahead of the step it folds, in
 // registers; one workgroup barrier per step stands for the exchange of the step's probabilities.  OCC workgroups per
-// CU.  What this reaches is what such a kernel could reach before its arithmetic.
+// CU.  (variant bits: 1 no barrier, 2 no scale loads, 4 V by tile.)  What this reaches is what such a kernel could reach before its arithmetic.
 template <int DEPTH, int OCC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_stream_probe_kernel(const PaDecodeArgs a, int* sink, int variant) {
@@ -117,7 +117,11 @@ void pa_stream_probe_kernel(const PaDecodeArgs a, int* sink, int variant) {
   const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
   const int last_tile_tok = (wg_end - 1) & ~15;
   const uint32_t k_off = (uint32_t)(kg * 256 + li * 16);
-  const uint32_t v_off = (uint32_t)((32 * wave + li) * 16);
+  // variant bit 2: wave w reads all 128 head dims of V for the step's tile w (what pa_partition_shared_kernel's
+  // waves fetch: 2 KiB in one piece) instead of 32 head dims for all four tiles (four pieces of 512 bytes)
+  const bool v_by_tile = variant & 4;
+  const uint32_t v_off = v_by_tile ? (uint32_t)(lane * 16) : (uint32_t)((32 * wave + li) * 16);
+  const uint32_t v_off2 = v_by_tile ? 1024u : 256u;
   struct Step {
     u32x4 k[2];
     u32x4 v[2];
@@ -141,9 +145,10 @@ void pa_stream_probe_kernel(const PaDecodeArgs a, int* sink, int variant) {
     vp = kg == 1 ? page[1] : vp;
     vp = kg == 2 ? page[2] : vp;
     vp = kg == 3 ? page[3] : vp;
+    vp = v_by_tile ? kp : vp;
     const char* vb = vbase + (int64_t)vp * a.stride_v_b;
     st.v[0] = load16_stream(vb + v_off);
-    st.v[1] = load16_stream(vb + v_off + 256);
+    st.v[1] = load16_stream(vb + v_off + v_off2);
     st.sc = __builtin_nontemporal_load(sc_lane + (int64_t)kp * sc_page_stride);
     __builtin_amdgcn_sched_barrier(0);
   };

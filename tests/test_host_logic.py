@@ -426,12 +426,16 @@ def test_launch_layer_choices(pa_lib):
         "pa_partition_kernel<fp8, strided, 4 waves> x 4096, sorted items"
     # c5: 64 rows per kv head over an FP8 cache with per-token scales
     assert info(b=256, hq=128, hkv=8, q=4, ctx=28856, ps=7424, per_token=True, ragged=True) == \
-        "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items"
+        "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items, " \
+        "an item's heads on one XCD"
     assert info(b=128, hq=64, hkv=4, q=2, ctx=4096, ps=4096) == \
         "pa_partition_shared_kernel<fp8, bs16, 2 ring slots, 4 workgroups per CU> x 512"
-    # ... whose grid is whole groups of eight (sequence, partition) items (an XCD takes every eighth, with all its heads)
-    assert info(b=3, hq=64, hkv=2, q=1, ctx=4096, ps=1024) == \
-        "pa_partition_shared_kernel<fp8, bs16, 2 ring slots, 4 workgroups per CU> x 32"
+    # per-token scales: the grid is whole groups of eight (sequence, partition) items (an XCD takes every eighth, with
+    # all its heads); 3 sequences x 4 partitions -> 16 items x 2 heads
+    assert info(b=3, hq=64, hkv=2, q=1, ctx=4096, ps=1024, per_token=True) == \
+        "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 32, an item's heads on one XCD"
+    assert info(b=3, hq=16, hkv=2, q=1, ctx=4096, ps=1024, per_token=True) == \
+        "pa_partition_kernel<fp8 per-token, bs16, 4 waves> x 32, an item's heads on one XCD"
     # c1: a bf16 cache, 8 rows, few workgroups
     assert info(b=4, hq=8, hkv=1, q=1, ctx=1024, ps=1024, kv="bf16") == "pa_partition_kernel<bf16, strided, 4 waves> x 4"
     # a bf16 cache with 32 rows per kv head: two row tiles per workgroup; ragged with a workspace: queued

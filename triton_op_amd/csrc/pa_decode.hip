@@ -151,10 +151,10 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     // workgroup per CU is worth more than a deeper ring (measured); with them it needs about 140
     c.waves = 4;
     c.per_cu = c.per_token ? 3 : 4;
-    // An XCD takes every eighth (sequence, partition) item with all its kv heads (the heads' per-token scales of a
+    // Per-token scales: an XCD takes every eighth (sequence, partition) item with all its kv heads (the heads' scales of a
     // page share 128-byte lines, which then meet in one L2; measured on the ragged 64-row mix: 341 -> 336 us, uniform
     // batches 1 %); the grid is whole groups of eight items.  PA_DECODE_XCD=0: the head fastest in the workgroup id.
-    c.heads_share_xcd = !xcd_off;
+    c.heads_share_xcd = c.per_token && !xcd_off;
     items = (long long)a.num_seqs * a.max_num_partitions;
     if (c.heads_share_xcd) items = (items + 7) / 8 * 8;
     items *= a.num_kv_heads;
@@ -549,16 +549,18 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
   if (!text || text_bytes <= 0) return PA_ERR_NULL_POINTER;
   const LaunchChoice c = choose_launch(*a);
   const char* cache = !c.fp8 ? "bf16" : (c.per_token ? "fp8 per-token" : "fp8");
+  const char* placed = c.heads_share_xcd ? ", an item's heads on one XCD" : "";
   if (c.shared)
-    snprintf(text, (size_t)text_bytes, "pa_partition_shared_kernel<%s, %s, %d ring slots, %d workgroups per CU> x %lld%s",
-             cache, c.bs16 ? "bs16" : "strided", c.per_token ? 3 : 2, c.per_cu, c.blocks, c.sorted ? ", sorted items" : "");
+    snprintf(text, (size_t)text_bytes, "pa_partition_shared_kernel<%s, %s, %d ring slots, %d workgroups per CU> x %lld%s%s",
+             cache, c.bs16 ? "bs16" : "strided", c.per_token ? 3 : 2, c.per_cu, c.blocks, c.sorted ? ", sorted items" : "",
+             placed);
   else
   {
     char span_text[48] = "";
     if (c.span > 1) snprintf(span_text, sizeof(span_text), ", %d partitions per workgroup", c.span);
-    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s%s", cache,
+    snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s%s%s", cache,
              c.bs16 ? "bs16" : "strided", c.waves, c.row_tiles == 2 ? ", 2 row tiles" : "", c.blocks,
-             c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""), span_text);
+             c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""), span_text, placed);
   }
   return PA_OK;
 }
