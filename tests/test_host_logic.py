@@ -105,7 +105,7 @@ def test_partition_size_from_the_longest_context_and_the_total():
     """The tuning layer's second statistic: the sum of the context lengths.  A batch counts as total / longest
     sequences of the longest length, so a batch whose tokens sit in one or two long sequences gets the small
     partitions of a small batch (measured on the GPU: 8 sequences, one of 65536 tokens and seven of 1024, 32 rows per
-    kv head: 132.6 us at 5632 against 51.5 us at 1536); an even batch, or no total, changes nothing."""
+    kv head: 106.7 us at 5632 against 49.6 us at 1536); an even batch, or no total, changes nothing."""
     f = T.select_partition_size
     # (num_seqs, kv heads, rows per group, longest context, block size, CUs, total tokens)
     assert f(8, 8, 32, 65536, 16, 256) == 5632 and f(8, 8, 32, 65536, 16, 256, 65536 + 7 * 1024) == 1536

@@ -196,7 +196,12 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1) * span;
     } else {
       b = (int)(item % a.num_seqs);
-      part = (int)(item / a.num_seqs) * span;
+      const int coarse = (int)(item / a.num_seqs);
+      part = coarse * span;
+      // (items go to the XCDs round robin: with a batch that is a multiple of eight every partition of a sequence
+      // would sit on the same XCD, and a batch's one long sequence on one eighth of the GPU; each partition index
+      // therefore starts the batch one sequence further on)
+      if (PER_TOKEN && (a.flags & kFlagHeadsShareXcd)) b = (b + coarse % a.num_seqs) % a.num_seqs;
     }
   }
   const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group

@@ -71,6 +71,10 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     if (item >= (long long)a.num_seqs * a.max_num_partitions) return;  // (the grid is whole groups of eight items)
     b = (int)(item % a.num_seqs);
     part = (int)(item / a.num_seqs);
+    // (items go to the XCDs round robin: with a batch that is a multiple of eight every partition of a sequence
+    // would sit on the same XCD, and a batch's one long sequence on one eighth of the GPU; each partition index
+    // therefore starts the batch one sequence further on)
+    if (a.flags & kFlagHeadsShareXcd) b = (b + part % a.num_seqs) % a.num_seqs;
   }
 
   const int ctx = sload_i32(a.context_lens + b);
