@@ -878,3 +878,26 @@ def test_many_partitions_of_few_rows_take_the_wide_reduce(cuda, group, q_len, ra
         merged = O.reduce_stage(plan.max_logits.cpu(), plan.exp_sums.cpu(), plan.tmp_output.float().cpu(), wl.context_lens, 256)
         torch.testing.assert_close(out.float().cpu(), merged.float(), atol=4e-3, rtol=8e-3)  # bf16 rounding only
     torch.testing.assert_close(out.float().cpu(), first.float().cpu(), atol=4e-3, rtol=8e-3)
+
+
+@pytest.mark.parametrize("num_q_heads,q_len,batch", [(16, 1, 8), (16, 1, 9), (32, 2, 8), (32, 4, 16)])
+def test_heads_of_an_item_on_one_xcd_in_plain_order(cuda, num_q_heads, q_len, batch):
+    """Per-token scales: workgroup ids are mapped so that an XCD takes every eighth (sequence, partition) item with
+    all its kv heads, the grid is padded to whole groups of eight items, and in plain (unsorted) order each partition
+    index starts the batch one sequence further on.  A skewed batch whose partition count exceeds the batch size
+    (the rotation wraps) and is not a multiple of eight, both partition kernels, stage-wise and end to end."""
+    import triton_op_amd as T
+
+    ctx = torch.full((batch,), 100, dtype=torch.int32)
+    ctx[1] = 256 * 11 - 7          # 11 partitions of 256: more than a batch of 8 or 9
+    ctx[batch - 1] = 700
+    wl = _make(batch=batch, num_q_heads=num_q_heads, num_kv_heads=2, context_lens=ctx, q_len=q_len, scale_mode="token")
+    g = wl.to(cuda)
+    info = T.plan_decode(torch.empty_like(g.query), g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                         g.softmax_scale, g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                         partition_size=256).launch_info()
+    assert "an item's heads on one XCD" in info and "sorted items" not in info, info
+    out, res = _run(wl, cuda, partition_size=256)
+    _check_stages(wl, res, 256)
+    ref = _oracle(wl)
+    assert torch.allclose(out.float(), ref.float(), atol=ATOL, rtol=RTOL)
