@@ -221,14 +221,23 @@ class _Config:
         self.wls = shared_from.wls if shared_from is not None else [
             _make_workload(name, dev, i, batch) for i in range(pools)]
         self.plans = []
+        # The KV pools rotate from call to call (a decode step reads every layer's cache once); the output, the
+        # partition buffers and the workspace are the same memory in every call, as in an engine that reuses its
+        # activation buffers from layer to layer (with buffers of their own per pool, c5's 70 MB of partial results
+        # and outputs per call cost it 5 %: re-written lines stay in the last-level cache, fresh ones go to HBM).
+        out = torch.empty(self.wls[0].query.shape, dtype=torch.bfloat16, device=dev)
+        shared = {}
         for wl in self.wls:
-            out = torch.empty(wl.query.shape, dtype=torch.bfloat16, device=dev)
             # the two context-length statistics a serving engine has on the host: the longest and the sum
-            self.plans.append(T.plan_decode(
+            plan = T.plan_decode(
                 out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
                 wl.q_len, wl.max_context_len, torch.bfloat16, wl.meta.get("query_scale"), wl.key_scale, wl.value_scale,
                 partition_size=partition_size or None, query_lens=wl.q_lens,
-                total_context_tokens=int(wl.context_lens.to(torch.int64).sum())))
+                total_context_tokens=int(wl.context_lens.to(torch.int64).sum()), **shared)
+            if not shared:
+                shared = dict(max_logits=plan.max_logits, exp_sums=plan.exp_sums, tmp_output=plan.tmp_output,
+                              workspace=plan.workspace)
+            self.plans.append(plan)
         self.wl0 = self.wls[0]
         self.kv_bytes = self.wl0.kv_bytes()
         self.partition_size = int(self.plans[0].args.partition_size)
