@@ -67,6 +67,11 @@ HBM_TRAFFIC = {
         "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items, "
                   "an item's heads on one XCD",
         "profile": "profiles/pa_partition_shared_kernel_c5_hbm_traffic.md"},
+    ("c5_ragged_mix", 7424, "output_only"): {
+        "bytes": 1_943_700_000,
+        "launch": "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 8192, sorted items, "
+                  "an item's heads on one XCD",
+        "profile": "profiles/pa_partition_shared_kernel_c5_hbm_traffic.md"},
 }
 
 
@@ -213,7 +218,7 @@ def _dtype_text(wl):
 class _Config:
     """`pools` independent copies of one workload with their validated plans."""
 
-    def __init__(self, name, dev, pools, partition_size=None, batch=None, shared_from=None):
+    def __init__(self, name, dev, pools, partition_size=None, batch=None, shared_from=None, output_only=False):
         import torch
 
         import triton_op_amd as T
@@ -233,7 +238,7 @@ class _Config:
                 out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
                 wl.q_len, wl.max_context_len, torch.bfloat16, wl.meta.get("query_scale"), wl.key_scale, wl.value_scale,
                 partition_size=partition_size or None, query_lens=wl.q_lens,
-                total_context_tokens=int(wl.context_lens.to(torch.int64).sum()), **shared)
+                total_context_tokens=int(wl.context_lens.to(torch.int64).sum()), output_only=output_only, **shared)
             if not shared:
                 shared = dict(max_logits=plan.max_logits, exp_sums=plan.exp_sums, tmp_output=plan.tmp_output,
                               workspace=plan.workspace)
@@ -241,6 +246,7 @@ class _Config:
         self.wl0 = self.wls[0]
         self.kv_bytes = self.wl0.kv_bytes()
         self.partition_size = int(self.plans[0].args.partition_size)
+        self.output_only = output_only
         self.launch = self.plans[0].launch_info()
         self.kernel = self.launch.split("<")[0]
 
@@ -380,7 +386,8 @@ def _sample_power(lib, cfg, stream, seconds):
 
 
 def _traffic(cfg):
-    entry = HBM_TRAFFIC.get((cfg.wl0.name, cfg.partition_size))
+    entry = HBM_TRAFFIC.get((cfg.wl0.name, cfg.partition_size, "output_only") if cfg.output_only
+                            else (cfg.wl0.name, cfg.partition_size))
     if entry is None:
         return None, "no rocprofv3 FETCH_SIZE/WRITE_SIZE measurement on record for this workload and partition size"
     if entry["launch"] != cfg.launch:
@@ -393,7 +400,9 @@ def _config_line(cfg, t):
     """The short record of a configuration for the `configs` array of the headline line."""
     achieved = cfg.kv_bytes / (t["kernel_us_avg"] * 1e-6) / 1e9
     return {
-        "workload": cfg.wl0.name, "partition_size": cfg.partition_size, "us_per_call": round(t["us_median"], 2),
+        "workload": cfg.wl0.name, "partition_size": cfg.partition_size,
+        # PA_DECODE_FLAG_OUTPUT_ONLY: the caller reads only the real query rows of `output` (include/pa_decode.h)
+        "output_only": cfg.output_only, "us_per_call": round(t["us_median"], 2),
         "kv_GBps": round(cfg.kv_bytes / (t["us_median"] * 1e-6) / 1e9, 1), "kernel": cfg.kernel, "launch": cfg.launch,
         "kernel_us_avg": round(t["kernel_us_avg"], 2), "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "reduce_us_avg": None if t["reduce_us_avg"] is None else round(t["reduce_us_avg"], 2),
@@ -469,7 +478,7 @@ def _bench_decode(a) -> int:
     stream = torch.cuda.current_stream(dev)
 
     headline = a.workload or "c2"
-    cfg = _Config(headline, dev, a.pools, a.partition_size, a.batch or None)
+    cfg = _Config(headline, dev, a.pools, a.partition_size, a.batch or None, output_only=a.output_only)
     t = _time_config(lib, cfg, stream, a.steps, a.warmup, a.settle)
     wl0 = cfg.wl0
     achieved = cfg.kv_bytes / (t["kernel_us_avg"] * 1e-6) / 1e9
@@ -533,6 +542,12 @@ def _bench_decode(a) -> int:
                 c4_256 = _Config("c4", dev, 1, 256, shared_from=other)
                 lines.append(_config_line(c4_256, _time_config(lib, c4_256, stream, min(a.steps, 30), 5, a.settle)))
                 del c4_256
+            if name == "c5":
+                # ... and as an engine calls it that reads only the real query rows of `output`: no partition-buffer
+                # entries for the sequences stage 1 finishes, no zeros for the rows beyond a sequence's query length
+                c5_lean = _Config("c5", dev, 1, shared_from=other, output_only=True)
+                lines.append(_config_line(c5_lean, _time_config(lib, c5_lean, stream, min(a.steps, 30), 5, a.settle)))
+                del c5_lean
             del other
             torch.cuda.empty_cache()
         result["configs"] = lines
@@ -785,6 +800,8 @@ def main() -> int:
     ap.add_argument("--workload", default="", help="default: c2 as the headline plus c2@256, c3, c4, c5 in `configs`")
     ap.add_argument("--partition-size", type=int, default=0, help="0 = let the tuning layer choose")
     ap.add_argument("--pools", type=int, default=3)
+    ap.add_argument("--output-only", action="store_true",
+                    help="call with PA_DECODE_FLAG_OUTPUT_ONLY (the caller reads only the real query rows of `output`)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="default run: the headline only")
     ap.add_argument("--power-seconds", type=float, default=0.0,

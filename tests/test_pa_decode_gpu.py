@@ -901,3 +901,52 @@ def test_heads_of_an_item_on_one_xcd_in_plain_order(cuda, num_q_heads, q_len, ba
     _check_stages(wl, res, 256)
     ref = _oracle(wl)
     assert torch.allclose(out.float(), ref.float(), atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("name", ["fp8_g8", "fp8_g16_q4", "fp8_token_ragged", "fp8_ragged_two_waves_per_tile",
+                                  "fp8_token_ragged_two_waves_per_tile", "bf16_ragged_g16_q4", "bf16_g16_q4",
+                                  "fp8_g8_q4_long", "fp8_bs1024_q2", "fp8_token_g8_q1"])
+@pytest.mark.parametrize("partition_size", [256, 1024, 4096])
+@pytest.mark.parametrize("with_sinks", [False, True])
+def test_output_only_flag(cuda, pa_lib, name, partition_size, with_sinks):
+    """PA_DECODE_FLAG_OUTPUT_ONLY: the caller reads only the real query rows of `output`.  Those rows equal the
+    flagless call's bit for bit (and so the oracle's, which that call is tested against); rows beyond a sequence's
+    query length are never NaN-poisoned into real rows; a sequence that stage 1 finishes leaves its padding rows as
+    they were and its partition-buffer entries untouched; the two stage entry points called one by one with the flag
+    give the same rows as pa_decode."""
+    import triton_op_amd as T
+
+    wl = _make(**CASES[name])
+    g = wl.to(cuda)
+    G = g.query.shape[1] // (g.q_len * g.key_cache.shape[1])
+    sinks = None
+    if with_sinks:
+        sinks = torch.linspace(-1.0, 1.0, g.query.shape[1], dtype=torch.float32, device=cuda)
+
+    def plan(out, **kw):
+        return T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                             g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                             partition_size=partition_size, query_lens=g.q_lens, sinks=sinks, **kw)
+
+    ref = torch.full_like(g.query, float("nan"))
+    plan(ref).run()
+    out = torch.full_like(g.query, 7.0)
+    p = plan(out, output_only=True)
+    p.exp_sums.fill_(-3.0)
+    p.run()
+    two = torch.full_like(g.query, 7.0)
+    p2 = plan(two, output_only=True)
+    p2.run_partition()
+    p2.run_reduce()
+    torch.cuda.synchronize()
+    Hkv, q_max = g.key_cache.shape[1], g.q_len
+    qls = g.q_lens.cpu().tolist() if g.q_lens is not None else [q_max] * g.query.shape[0]
+    ctxs = g.context_lens.cpu().tolist()
+    view = lambda t: t.view(t.shape[0], Hkv, q_max, G, -1)
+    for b, (ql, ctx) in enumerate(zip(qls, ctxs)):
+        live = (view(out)[b, :, :ql], view(two)[b, :, :ql], view(ref)[b, :, :ql])
+        assert torch.equal(live[0], live[2]) and torch.equal(live[1], live[2]), f"sequence {b}"
+        finished_by_stage_1 = (ctx <= partition_size or p.max_logits.shape[2] == 1) and sinks is None
+        if finished_by_stage_1 and ctx > 0:
+            assert torch.all(view(out)[b, :, ql:] == 7.0), f"padding rows of sequence {b} were written"
+            assert torch.all(p.exp_sums[b] == -3.0), f"partition-buffer entries of sequence {b} were written"

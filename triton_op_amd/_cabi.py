@@ -17,6 +17,7 @@ PA_DECODE_WORKSPACE_BYTES = 64
 PA_DECODE_NOALLOC_SCRATCH_BYTES = 64 << 20
 PA_ERR_SCRATCH_TOO_SMALL = -7
 PA_DECODE_FLAG_REUSE_ITEM_LIST = 1
+PA_DECODE_FLAG_OUTPUT_ONLY = 2
 PA_DTYPE_BF16, PA_DTYPE_FP8_E4M3FN = 0, 1
 PA_QUANT_NONE, PA_QUANT_PER_TENSOR, PA_QUANT_PER_TOKEN = -1, 0, 1
 

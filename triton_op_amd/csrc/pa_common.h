@@ -22,6 +22,9 @@ typedef __attribute__((ext_vector_type(8))) int i32x8;
 constexpr int kHeadSize = 128;
 // PaDecodeArgs.flags as the kernels see it (the launch layer sets it in its own copy of the arguments)
 constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning kernel's item list
+// PA_DECODE_FLAG_OUTPUT_ONLY as the kernels see it: no partition-buffer entries for a sequence this stage finishes,
+// nothing written for rows beyond a sequence's query length
+constexpr int kFlagOutputOnly = 0x20000;
 constexpr int kFlagSpanShift = 20;         // bits 20..27: partitions a one-wave workgroup walks in one pass (0 = 1)
 // experiment switch of pa_partition_shared_kernel: P without its FP8 residual
 constexpr int kFlagResidualNever = 0x40000;

@@ -58,7 +58,7 @@ int check_common(const PaDecodeArgs* a) {
       a->max_num_partitions <= 0)
     return PA_ERR_BAD_SHAPE;
   if (a->partition_size <= 0 || a->partition_size % 256) return PA_ERR_BAD_SHAPE;
-  if (a->flags & ~PA_DECODE_FLAG_REUSE_ITEM_LIST) return PA_ERR_BAD_SHAPE;
+  if (a->flags & ~(PA_DECODE_FLAG_REUSE_ITEM_LIST | PA_DECODE_FLAG_OUTPUT_ONLY)) return PA_ERR_BAD_SHAPE;
   if (a->workspace ? a->workspace_bytes < PA_DECODE_WORKSPACE_BYTES : a->workspace_bytes != 0) return PA_ERR_BAD_SHAPE;
   if (a->head_size != kHeadSize) return PA_ERR_UNSUPPORTED;
   if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;  // the reference's limit
@@ -301,6 +301,7 @@ int launch_partition(const PaDecodeArgs& a, const LaunchChoice& c, hipStream_t s
   }
   if (c.span > 1) k.flags |= c.span << kFlagSpanShift;
   if (c.heads_share_xcd) k.flags |= kFlagHeadsShareXcd;
+  if (a.flags & PA_DECODE_FLAG_OUTPUT_ONLY) k.flags |= kFlagOutputOnly;
   // experiment (PA_DECODE_DEBUG=1): PA_DECODE_P_RESIDUAL=0 drops the FP8 residual of P in the shared-stream kernel
   // (every P rounded to e4m3, as the reference's kernel rounds it)
   static const int p_residual = debug_switch("PA_DECODE_P_RESIDUAL", 1);
@@ -527,7 +528,16 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
   return launch_partition(*a, choose_launch(*a), reinterpret_cast<hipStream_t>(hip_stream));
 }
 
-int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) { return launch_reduce(a, hip_stream, false); }
+int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
+  // PA_DECODE_FLAG_OUTPUT_ONLY: stage 1 ran with the same flag and left no entries for the sequences it finished
+  // itself; stage 2 passes over them, as it does inside pa_decode
+  const bool lean = a && a->struct_size == sizeof(PaDecodeArgs) && (a->flags & PA_DECODE_FLAG_OUTPUT_ONLY);
+  if (lean && a->max_num_partitions == 1 && !a->sinks) {
+    const int rc = check_reduce(a);
+    return rc;  // every sequence was finished by stage 1
+  }
+  return launch_reduce(a, hip_stream, lean);
+}
 
 int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
   int rc = check_partition(a);

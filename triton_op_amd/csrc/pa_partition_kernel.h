@@ -234,7 +234,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int rows_valid = qb * G;
   if (row0 >= rows_valid) {
     // only padding rows (a ragged batch): nothing to stream; the rows read as "no visible key"
-    if (wave == 0) {
+    if (wave == 0 && !(a.flags & kFlagOutputOnly)) {
       auto write_padding = [&](int pp) {
         const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)pp * a.stride_es_p;
         char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
@@ -817,6 +817,11 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // cuts off longer contexts for any other length.)
   const bool direct = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+  // PA_DECODE_FLAG_OUTPUT_ONLY: rows beyond the sequence's query length are nobody's, and a sequence finished here
+  // leaves no partition-buffer entries
+  const bool output_only = a.flags & kFlagOutputOnly;
+  const bool no_partial = output_only && direct;
+  const int rows_live = output_only ? rows_valid : Ge;
   float l_tot[NT], acc_unit[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -832,15 +837,20 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     for (int nt = 0; nt < NT; ++nt) {
       const int row = row0 + 16 * nt + li;
       const float inv = l_tot[nt] > 0.f ? v_tensor_scale * acc_unit[nt] / l_tot[nt] : 0.f;
-      if (row < Ge && kg == 0) {
+      if (row < rows_live && kg == 0 && !no_partial) {
         a.max_logits[es_off + row] = m_run[nt] * (1.0f / kLog2e);
         a.exp_sums[es_off + row] = l_tot[nt];
       }
       // (one-wave workgroups stage the last partition's tile in the next free slot of the pool)
       char* stage_at = kSpanCapable ? &span_lds[0] + ((part_cur - part) * NT + nt) * span_slot_bytes : &o_lds[0][0];
-      store_partial_tile(stage_at, acc[nt], inv, tmp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2,
-                         a.stride_tmp_g * 2, direct ? outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2 : nullptr,
-                         a.stride_out_h * 2, Ge - row0 - 16 * nt, lane, kSpanCapable ? span_rows : 16);
+      char* out_tile = outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2;
+      if (no_partial)
+        store_partial_tile(stage_at, acc[nt], inv, out_tile, a.stride_out_h * 2, nullptr, 0, rows_live - row0 - 16 * nt,
+                           lane, kSpanCapable ? span_rows : 16);
+      else
+        store_partial_tile(stage_at, acc[nt], inv, tmp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2,
+                           a.stride_tmp_g * 2, direct ? out_tile : nullptr, a.stride_out_h * 2, rows_live - row0 - 16 * nt,
+                           lane, kSpanCapable ? span_rows : 16);
     }
   } else {
     // merge the waves' (m, l, O): every wave holds the same (row, head dim) in the same lane and register,
@@ -887,7 +897,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         pk[1] = pack_bf16x2(o[2], o[3]);
         *reinterpret_cast<u32x2*>(&o_lds[0][0] + li * kORowBytes + (16 * db + 4 * kg) * 2) = pk;
       }
-      if (wave == 0 && kg == 0 && row < Ge) {
+      if (wave == 0 && kg == 0 && row < rows_live && !no_partial) {
         a.max_logits[es_off + row] = M * (1.0f / kLog2e);
         a.exp_sums[es_off + row] = L;
       }
@@ -895,8 +905,8 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       for (int i = wave; i < 4; i += WAVES) {
         const int r = 4 * i + kg;
         const u32x4 v = *reinterpret_cast<const u32x4*>(&o_lds[0][0] + r * kORowBytes + li * 16);
-        if (r < Ge - row0 - 16 * nt) {
-          *reinterpret_cast<u32x4*>(tmp + (int64_t)(row0 + 16 * nt + r) * a.stride_tmp_g * 2 + li * 16) = v;
+        if (r < rows_live - row0 - 16 * nt) {
+          if (!no_partial) *reinterpret_cast<u32x4*>(tmp + (int64_t)(row0 + 16 * nt + r) * a.stride_tmp_g * 2 + li * 16) = v;
           if (direct)
             *reinterpret_cast<u32x4*>(outp + (int64_t)(row0 + 16 * nt + r) * a.stride_out_h * 2 + li * 16) = v;
         }
@@ -915,18 +925,18 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       for (int nt = 0; nt < NT; ++nt) {
         const char* slot = &span_lds[0] + ((pc - part) * NT + nt) * span_slot_bytes;
         const int row = row0 + 16 * nt + li;
-        if (row < Ge && kg == 0) {
+        if (row < rows_live && kg == 0) {
           a.max_logits[eo + row] = reinterpret_cast<const float*>(slot + span_rows * kORowBytes)[li];
           a.exp_sums[eo + row] = reinterpret_cast<const float*>(slot + span_rows * kORowBytes)[16 + li];
         }
         copy_staged_tile(slot, tp + (int64_t)(row0 + 16 * nt) * a.stride_tmp_g * 2, a.stride_tmp_g * 2, nullptr, 0,
-                         Ge - row0 - 16 * nt, lane);
+                         rows_live - row0 - 16 * nt, lane);
       }
     }
   }
   if constexpr (QUEUE) {
     // rows of padding query positions beyond the last real tile: this workgroup fills them
-    if (rt == tiles_b - 1 && wave == 0) {
+    if (rt == tiles_b - 1 && wave == 0 && !output_only) {
       for (int r = 16 * NT * tiles_b + kg; r < Ge; r += 4) {
         if (li == 0) {
           a.max_logits[es_off + r] = -INFINITY;

@@ -540,7 +540,9 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   __syncthreads();  // the stage buffers are free
 
   // a tile of padding rows only (a ragged batch): the rows read as "no visible key"
+  const bool output_only = a.flags & kFlagOutputOnly;
   auto write_padding_rows = [&](int first_row) {
+    if (output_only) return;  // nobody reads them (the merge of a longer sequence writes what it finds to rows nobody reads)
     for (int r = first_row + kg; r < first_row + 16 && r < Ge; r += 4) {
       if (li == 0) {
         a.max_logits[es_off + r] = -INFINITY;
@@ -608,7 +610,8 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     m_true = -INFINITY;
   }
   const float inv = l_tot > 0.f ? v_tensor_scale * acc_unit / l_tot : 0.f;
-  if (row < Ge && kg == 0) {
+  const bool no_partial = output_only && direct;  // finished here: nobody merges this sequence
+  if (row < Ge && kg == 0 && !no_partial) {
     // the partition buffers hold the true maximum and the sum taken against it
     a.max_logits[es_off + row] = m_true * (1.0f / kLog2e);
     a.exp_sums[es_off + row] = l_tot > 0.f ? l_tot * fast_exp2(m_ref - m_true) : 0.f;
@@ -616,8 +619,13 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   // wave-private staging for the transposed store (two waves per tile: behind the merge buffers, one per tile)
   char* olds = reinterpret_cast<char*>(&stage[0]) +
                (half_mode ? 2 * (3 * 16 + 32 * 64) * 4 + (row0 >> 4) * (16 * kORowBytes) : wave * (16 * kORowBytes));
-  store_partial_tile(olds, acc, inv, tmp + (int64_t)row0 * a.stride_tmp_g * 2, a.stride_tmp_g * 2,
-                     direct ? outp + (int64_t)row0 * a.stride_out_h * 2 : nullptr, a.stride_out_h * 2, Ge - row0, lane);
+  const int rows_out = (output_only ? rows_valid : Ge) - row0;
+  if (no_partial)
+    store_partial_tile(olds, acc, inv, outp + (int64_t)row0 * a.stride_out_h * 2, a.stride_out_h * 2, nullptr, 0,
+                       rows_out, lane);
+  else
+    store_partial_tile(olds, acc, inv, tmp + (int64_t)row0 * a.stride_tmp_g * 2, a.stride_tmp_g * 2,
+                       direct ? outp + (int64_t)row0 * a.stride_out_h * 2 : nullptr, a.stride_out_h * 2, rows_out, lane);
 }
 
 }  // namespace

@@ -103,7 +103,7 @@ class DecodePlan:
         a = PaDecodeArgs.from_buffer_copy(self.args)
         a.exp_sums = a.max_logits = a.tmp_output = a.workspace = None
         a.workspace_bytes = 0
-        a.flags = 0
+        a.flags &= _cabi.PA_DECODE_FLAG_OUTPUT_ONLY
         _cabi.check(self._lib.pa_decode_noalloc(C.byref(a), C.c_void_p(stream)), "pa_decode_noalloc")
 
     def run_partition(self, stream: Optional[int] = None) -> None:
@@ -144,6 +144,7 @@ def plan_decode(
     sinks: Optional[torch.Tensor] = None,
     reuse_item_list: bool = False,
     total_context_tokens: int = 0,
+    output_only: bool = False,
 ) -> DecodePlan:
     if temp_output is not None:  # the spelling of run_gluon_fp8_kernel (test_pa_mtp.py:566-584)
         if tmp_output is not None and tmp_output is not temp_output:
@@ -357,7 +358,8 @@ def plan_decode(
     a.workspace_bytes = workspace.numel() * 4
     # the caller's word that `workspace` already holds the item list of a call with the same sequence lengths
     # and partitioning (the previous layer of this decode step): the planning kernel is skipped
-    a.flags = _cabi.PA_DECODE_FLAG_REUSE_ITEM_LIST if reuse_item_list else 0
+    a.flags = (_cabi.PA_DECODE_FLAG_REUSE_ITEM_LIST if reuse_item_list else 0) | \
+        (_cabi.PA_DECODE_FLAG_OUTPUT_ONLY if output_only else 0)
     a.num_seqs, a.num_kv_heads, a.group_size, a.q_len = num_seqs, num_kv_heads, group, q_len
     a.head_size, a.block_size = head_size, block_size
     a.max_num_partitions, a.partition_size = max_parts, partition_size
@@ -405,15 +407,18 @@ def paged_attention_decode(
     sinks: Optional[torch.Tensor] = None,
     reuse_item_list: bool = False,
     total_context_tokens: int = 0,
+    output_only: bool = False,
 ) -> Dict[str, object]:
     """Split-KV paged-attention decode; writes `output` in place on torch's current stream and
-    returns the partition buffers under the reference's keys."""
+    returns the partition buffers under the reference's keys.  `output_only=True` (PA_DECODE_FLAG_OUTPUT_ONLY): the
+    caller reads nothing but the rows of `output` that belong to real query rows; the partition buffers are scratch
+    with unspecified contents afterwards, and rows beyond a sequence's `query_lens` entry are left as they were."""
     plan = plan_decode(
         output, query, key_cache, value_cache, sequence_lengths, block_tables, softmax_scale,
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
         num_sequence_partitions, alibi_slopes, max_logits, exp_sums, tmp_output, temp_output=temp_output,
         partition_size=partition_size, query_lens=query_lens, workspace=workspace,
-        sinks=sinks, reuse_item_list=reuse_item_list, total_context_tokens=total_context_tokens)
+        sinks=sinks, reuse_item_list=reuse_item_list, total_context_tokens=total_context_tokens, output_only=output_only)
     plan.run()
     return {
         "temporary_output": plan.tmp_output,
