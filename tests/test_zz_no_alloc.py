@@ -115,3 +115,22 @@ def test_noalloc_refuses_what_does_not_fit():
     assert rc == _cabi.PA_ERR_SCRATCH_TOO_SMALL
     torch.cuda.synchronize()
     assert torch.equal(out, torch.full_like(out, 7.0))  # nothing ran
+
+
+def test_noalloc_with_the_output_only_flag():
+    """PA_DECODE_FLAG_OUTPUT_ONLY through the entry point that allocates nothing: the real query rows equal
+    pa_decode's bit for bit."""
+    dev = torch.device("cuda:0")
+    wl, ps = _workloads(dev)[0]
+    ref = torch.full_like(wl.query, float("nan"))
+    _plan(wl, ref, ps).run()
+    out = torch.full_like(wl.query, 7.0)
+    plan = T.plan_decode(out, wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables,
+                         wl.softmax_scale, wl.q_len, wl.max_context_len, torch.bfloat16, None, wl.key_scale,
+                         wl.value_scale, partition_size=ps, query_lens=wl.q_lens, output_only=True)
+    plan.run_noalloc(torch.cuda.current_stream(dev).cuda_stream)
+    torch.cuda.synchronize()
+    hkv = wl.key_cache.shape[1]
+    view = lambda t: t.view(t.shape[0], hkv, wl.q_len, -1, t.shape[-1])
+    for b, ql in enumerate(wl.q_lens.cpu().tolist()):
+        assert torch.equal(view(out)[b, :, :ql], view(ref)[b, :, :ql]), f"sequence {b}"
