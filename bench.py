@@ -12,6 +12,7 @@
     python bench.py --workload probe_stream42:c5                     the pages read by workgroups whose waves share each step
                                                                      (depth 4 steps in registers, 2 workgroups per CU)
     python bench.py --workload probe_issue                           issue cost of the decode step's instructions
+    python bench.py --workload trace:c5                              where a workgroup slot's time goes (measuring build)
     python bench.py --workload kv_write | kv_quantize                the KV-cache write kernels, the step before the path
 
 A step is one call of the op (partition kernel + reduce kernel on one stream) on one batch of synthetic input
@@ -639,6 +640,74 @@ def _bench_probe_gather(a) -> int:
     return 0
 
 
+def _bench_trace(a) -> int:
+    """`--workload trace:W`: W (a workload of pa_partition_shared_kernel) through the measuring build of the library
+    (tests/native/libpa_decode_trace.so, -DPA_DECODE_TRACE): one wave of every workgroup leaves timestamps of the
+    100 MHz wall clock at its entry, after it has requested its first steps, when its query operands are ready, when
+    the first step has landed, after its last step and at its end.  Prints where a workgroup slot's time goes."""
+    here = os.path.dirname(os.path.abspath(__file__))
+    os.environ["PA_DECODE_LIB"] = os.path.join(here, "tests", "native", "libpa_decode_trace.so")  # before the first load
+    import numpy as np
+    import torch
+
+    from triton_op_amd import _cabi
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    lib = _cabi.load_library()
+    lib.pa_decode_trace_read.argtypes = [C.c_void_p, C.c_ulonglong]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream(dev)
+    sh = C.c_void_p(stream.cuda_stream)
+    cfg = _Config(a.workload.partition(":")[2] or "c5", dev, 1, a.partition_size, a.batch or None, output_only=a.output_only)
+    if cfg.kernel != "pa_partition_shared_kernel":
+        print(f"trace: only pa_partition_shared_kernel leaves timestamps; this workload launches {cfg.launch}", file=sys.stderr)
+        return 2
+    plan = cfg.plans[0]
+    for _ in range(a.settle):
+        _cabi.check(lib.pa_decode(C.byref(plan.args), sh), "pa_decode")
+    torch.cuda.synchronize()
+    _cabi.check(lib.pa_decode_trace_clear(), "pa_decode_trace_clear")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    _cabi.check(lib.pa_decode(C.byref(plan.args), sh), "pa_decode")
+    e1.record(stream)
+    torch.cuda.synchronize()
+    words = np.zeros(16384 * 8, dtype=np.uint64)
+    _cabi.check(lib.pa_decode_trace_read(words.ctypes.data, words.nbytes), "pa_decode_trace_read")
+    t = words.reshape(-1, 8).astype(np.float64)
+    t = t[t[:, 5] > 0]
+    us = 0.01  # per tick
+    ent, req, qry, first, last, end, steps, rows = [t[:, i] for i in range(8)]
+    start, span = ent.min(), (end.max() - ent.min()) * us
+    slots = int(plan.launch_info().split(" workgroups per CU")[0].split()[-1]) * torch.cuda.get_device_properties(dev).multi_processor_count
+
+    def stat(x):
+        return {"mean_us": round(float(x.mean() * us), 2), "p10_us": round(float(np.percentile(x, 10) * us), 2),
+                "p90_us": round(float(np.percentile(x, 90) * us), 2), "per_slot_us": round(float(x.sum() * us / slots), 1)}
+
+    ev = np.concatenate([np.stack([ent, np.ones_like(ent)], 1), np.stack([end, -np.ones_like(end)], 1)])
+    ev = ev[np.argsort(ev[:, 0], kind="stable")]
+    active, when = np.cumsum(ev[:, 1]), (ev[:, 0] - start) * us
+    tail_from = float(when[np.where(active >= 0.9 * slots)[0][-1]]) if (active >= 0.9 * slots).any() else 0.0
+    print(json.dumps({
+        "metric": "where a workgroup slot's time goes (per-workgroup timestamps, measuring build)", "workload": cfg.wl0.name,
+        "launch": cfg.launch, "call_us": round(e0.elapsed_time(e1) * 1e3, 1), "live_workgroups": int(len(t)),
+        "workgroup_slots": slots, "launch_span_us": round(float(span), 1),
+        "entry_to_first_steps_requested": stat(req - ent), "entry_to_query_ready": stat(qry - ent),
+        "entry_to_first_step_landed": stat(first - ent), "main_loop": stat(last - first),
+        "per_step_in_loop": stat((last - first) / np.maximum(steps, 1)), "epilogue": stat(end - last),
+        "whole_workgroup": stat(end - ent),
+        "slot_time_used": round(float((end - ent).sum() * us / (slots * span)), 3),
+        "last_time_nine_tenths_of_the_slots_are_busy_us": round(tail_from, 1),
+        "per_step_us_by_live_rows": {str(r): round(float((((last - first) / steps)[(rows > r - 16) & (rows <= r) & (steps >= 16)]).mean() * us), 2)
+                                     for r in (16, 32, 48, 64) if ((rows > r - 16) & (rows <= r) & (steps >= 16)).any()},
+    }, ensure_ascii=False))
+    return 0
+
+
 def _bench_probe_issue(a) -> int:
     """What the instructions of the decode step cost a SIMD's issue port (pa_probe_issue): nanoseconds per
     instruction per wave with one and with three waves on every SIMD, and how far the matrix pipe runs beside the
@@ -818,6 +887,8 @@ def main() -> int:
         return _bench_kv_cache(a)
     if a.workload.partition(":")[0] == "probe_gather" or a.workload.startswith("probe_stream"):
         return _bench_probe_gather(a)
+    if a.workload.startswith("trace:") or a.workload == "trace":
+        return _bench_trace(a)
     if a.workload == "probe_issue":
         return _bench_probe_issue(a)
     return _bench_decode(a)

@@ -85,6 +85,21 @@ def build_probe(verbose: bool = True) -> str:
     return PROBE_LIB
 
 
+TRACE_LIB = os.path.join(HERE, "..", "tests", "native", "libpa_decode_trace.so")
+
+
+def build_trace(verbose: bool = True) -> str:
+    """The measuring build of the decode library (-DPA_DECODE_TRACE): the same sources, with per-workgroup timestamps
+    in pa_partition_shared_kernel, for bench.py's `trace:` workloads.  Never loaded by the product path."""
+    cmd = [find_hipcc(), *HIPCC_FLAGS, "-DPA_DECODE_TRACE", *SOURCES, "-o", TRACE_LIB]
+    if verbose:
+        print("[triton_op_amd.build]", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
+    return TRACE_LIB
+
+
 def is_stale() -> bool:
     if not os.path.exists(LIB_PATH):
         return True
@@ -96,3 +111,4 @@ if __name__ == "__main__":
     build()
     build_native_smoke()
     build_probe()
+    build_trace()

@@ -19,6 +19,19 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 
+// -DPA_DECODE_TRACE (the measuring build tests/native/libpa_decode_trace.so, never the product library): one wave of
+// every workgroup of pa_partition_shared_kernel leaves six timestamps of the 100 MHz wall clock, its step count
+// and its live rows in pa_trace; pa_decode_trace_read copies them out.  PA_TRACE_MARK(i) is nothing otherwise.
+#ifdef PA_DECODE_TRACE
+constexpr int kTraceWorkgroups = 16384;
+__device__ unsigned long long pa_trace[kTraceWorkgroups * 8];
+#define PA_TRACE_DECL unsigned long long pa_trace_t[6] = {0, 0, 0, 0, 0, 0}
+#define PA_TRACE_MARK(i) pa_trace_t[i] = wall_clock64()
+#else
+#define PA_TRACE_DECL
+#define PA_TRACE_MARK(i)
+#endif
+
 constexpr int kHeadSize = 128;
 // PaDecodeArgs.flags as the kernels see it (the launch layer sets it in its own copy of the arguments)
 constexpr int kFlagSortedItems = 0x10000;  // the workspace holds the planning kernel's item list

@@ -411,6 +411,20 @@ int launch_reduce_listed(const PaDecodeArgs* a, void* hip_stream) {
 }  // namespace
 
 extern "C" {
+#ifdef PA_DECODE_TRACE
+// the measuring build only: the workgroups' timestamps of the last pa_partition_shared_kernel launch (8 words per
+// workgroup id; workgroups that exited at once, or never ran, leave what was there: clear with pa_decode_trace_clear)
+int pa_decode_trace_read(void* dst, unsigned long long bytes) {
+  if (bytes > sizeof(pa_trace)) return PA_ERR_BAD_SHAPE;
+  return hipMemcpyFromSymbol(dst, HIP_SYMBOL(pa_trace), bytes) == hipSuccess ? PA_OK : PA_ERR_LAUNCH;
+}
+int pa_decode_trace_clear(void) {
+  void* p = nullptr;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(pa_trace)) != hipSuccess) return PA_ERR_LAUNCH;
+  return hipMemset(p, 0, sizeof(pa_trace)) == hipSuccess ? PA_OK : PA_ERR_LAUNCH;
+}
+#endif
+
 
 int pa_decode_abi_version(void) { return PA_DECODE_ABI_VERSION; }
 uint32_t pa_decode_args_size(void) { return (uint32_t)sizeof(PaDecodeArgs); }

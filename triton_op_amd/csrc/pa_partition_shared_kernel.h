@@ -36,6 +36,8 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   static_assert(sizeof(StepLds) * NB <= 65536, "the LDS address of an asynchronous load travels in 16 bits of M0");
   constexpr int kLoadsPerStep = PER_TOKEN ? 5 : 4;  // vector memory operations one wave issues per step
 
+  PA_TRACE_DECL;
+  PA_TRACE_MARK(0);  // entry
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15;
@@ -184,6 +186,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     }
   }
 
+  PA_TRACE_MARK(1);  // the first steps are requested
   // ---- buffers of this item ---------------------------------------------------------------------------------
   const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
   char* tmp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
@@ -267,6 +270,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     }
   }
 
+  PA_TRACE_MARK(2);  // the query operands are ready
   const bool rs_nonneg = __builtin_amdgcn_ballot_w64(rscale < 0.f) == 0;
   // Online softmax against a reference that (almost) never moves.  l and the accumulator are kept relative to
   // m_ref, the row's maximum at its first visible step, and in units of 2^k_ref (per-token V scales: the exponent
@@ -490,6 +494,9 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
       dma_wait<0>();
     // everybody's quarter of step s is in LDS, and everybody is done reading step s-1, whose slot is refilled now
     __syncthreads();
+#ifdef PA_DECODE_TRACE
+    if (s == 0) PA_TRACE_MARK(3);  // the first step has landed
+#endif
     if (s + NB - 1 < n_steps) {
       fetch(fetch_slot, pg_next);
       fetch_tok += kStepTokens;
@@ -538,6 +545,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     }
   }
   __syncthreads();  // the stage buffers are free
+  PA_TRACE_MARK(4);  // the last step is done
 
   // a tile of padding rows only (a ragged batch): the rows read as "no visible key"
   const bool output_only = a.flags & kFlagOutputOnly;
@@ -626,6 +634,16 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   else
     store_partial_tile(olds, acc, inv, tmp + (int64_t)row0 * a.stride_tmp_g * 2, a.stride_tmp_g * 2,
                        direct ? outp + (int64_t)row0 * a.stride_out_h * 2 : nullptr, a.stride_out_h * 2, rows_out, lane);
+#ifdef PA_DECODE_TRACE
+  if (lane == 0 && row0 == 0 && half == 0 && blockIdx.x < kTraceWorkgroups) {  // (these waves run to the end)
+    unsigned long long* t = pa_trace + 8ull * blockIdx.x;
+#pragma unroll
+    for (int i = 0; i < 5; ++i) t[i] = pa_trace_t[i];
+    t[5] = wall_clock64();
+    t[6] = (unsigned long long)n_steps;
+    t[7] = (unsigned long long)rows_valid;
+  }
+#endif
 }
 
 }  // namespace
