@@ -66,9 +66,14 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   int b, part;
   if (a.flags & kFlagSortedItems) {
     // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
-    if (item >= sload_i32(a.workspace + 2)) return;
-    b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);
-    part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1);
+    // (the number of listed items and this item's record are requested together: the list area is sized for every
+    // (sequence, partition) pair, and the grid's padding items read the last record)
+    const long long pairs = (long long)a.num_seqs * a.max_num_partitions;
+    const long long rec = item < pairs ? item : pairs - 1;
+    const int listed = sload_i32(a.workspace + 2);
+    b = sload_i32(a.workspace + kPlanHeaderWords + 2 * rec);
+    part = sload_i32(a.workspace + kPlanHeaderWords + 2 * rec + 1);
+    if (item >= listed) return;
   } else {
     if (item >= (long long)a.num_seqs * a.max_num_partitions) return;  // (the grid is whole groups of eight items)
     b = (int)(item % a.num_seqs);
@@ -79,6 +84,19 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     if (a.flags & kFlagHeadsShareXcd) b = (b + part % a.num_seqs) % a.num_seqs;
   }
 
+  // The block-table entries of this wave's tile of the first NB-1 steps are requested together with the context
+  // length, not after it (every dependent scalar load is a round trip under full memory load, and three of them in
+  // a row were 4 us before a workgroup's first request went out).  They are entries of this sequence's row (the
+  // index is kept inside the row); one that lies beyond the sequence's end is read but never used.
+  const int log2_bs = 31 - __builtin_clz(a.block_size);
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  int early_page[NB - 1];
+#pragma unroll
+  for (int i = 0; i < NB - 1; ++i) {
+    int idx = (part * a.partition_size + i * kStepTokens + 16 * wave) >> log2_bs;
+    idx = idx < (int)a.stride_bt_s ? idx : (int)a.stride_bt_s - 1;
+    early_page[i] = sload_i32(bt + idx);
+  }
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;
   if (wg_start >= ctx) {
@@ -105,7 +123,6 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const bool has_rows = row0 < rows_valid;  // else the wave only helps to fetch
 
   // ---- cache addressing ----------------------------------------------------------------------------------
-  const int log2_bs = 31 - __builtin_clz(a.block_size);
   const int bs_mask = a.block_size - 1;
   const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h;
   const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h;
@@ -126,7 +143,6 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   for (int i = 0; i < 2; ++i) v_lane_off[i] = (uint32_t)(lane + 64 * i) * v_row_bytes;
   const float* sc_lane = PER_TOKEN ? ((lane & 16) ? vsbase : ksbase) + li : nullptr;
 
-  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
   const int last_tile_tok = (wg_end - 1) & ~15;
   // wave w fetches tile w of every step: its page id (a scalar load) and the tile's token offset inside the
   // page.  Tiles past the last live one repeat it, so no block-table slot or page beyond the sequence is touched.
@@ -175,16 +191,23 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   };
 
   // ---- the first NB-1 steps go out before anything else is set up ----------------------------------------------
-  TilePage pg_next = load_page(wg_start);  // of the next step to fetch
   int fetch_tok = wg_start;
 #pragma unroll
   for (int i = 0; i < NB - 1; ++i) {
     if (i < n_steps) {
-      fetch(i, pg_next);
+      const int t = fetch_tok + 16 * wave;
+      TilePage tp;
+      if (t <= last_tile_tok) {  // (the early request was for this tile)
+        tp.page = early_page[i];
+        tp.off = t & bs_mask;
+      } else {
+        tp = load_page(fetch_tok);
+      }
+      fetch(i, tp);
       fetch_tok += kStepTokens;
-      pg_next = load_page(fetch_tok);
     }
   }
+  TilePage pg_next = load_page(fetch_tok);  // of the next step to fetch
 
   PA_TRACE_MARK(1);  // the first steps are requested
   // ---- buffers of this item ---------------------------------------------------------------------------------
