@@ -207,6 +207,19 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
   do {  // the body of one item; `break` leaves it
 
+  // The block-table entries of this wave's first step are requested together with the context length, not after it
+  // (dependent scalar loads are round trips under full memory load; the first request of a workgroup waits for
+  // all of them).  They are entries of this sequence's row (the index is kept inside the row); one that lies beyond
+  // the sequence's end is read but never used.
+  const int log2_bs = 31 - __builtin_clz(a.block_size);
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  int early_page[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int idx = (part * a.partition_size + wave * kStepTokens + 16 * j) >> log2_bs;
+    idx = idx < (int)a.stride_bt_s ? idx : (int)a.stride_bt_s - 1;
+    early_page[j] = sload_i32(bt + idx);
+  }
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;
   if (wg_start >= ctx) {
@@ -260,7 +273,6 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   }
 
   // ---- cache addressing -------------------------------------------------------------------------------
-  const int log2_bs = 31 - __builtin_clz(a.block_size);
   const int bs_mask = a.block_size - 1;
   const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h * esz;
   const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h * esz;
@@ -285,7 +297,6 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 #pragma unroll
   for (int db = 0; db < 8; ++db) v_lane_off[db] = li * v_row_bytes + 16 * db * v_row_bytes;
 
-  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
   const int last_tile_tok = (wg_end - 1) & ~15;  // first token of the last tile that holds a live token
 
   // page ids of the four tiles of the step that starts at token tok0 (scalar loads; tiles past the
@@ -357,7 +368,16 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int n_steps = active ? (wg_steps - wave + WAVES - 1) / WAVES : 0;
   SD buf_a;  // one step of cache data, refilled in place for the next step
   if (active) {
-    Pages pg0 = load_pages(part_start);
+    Pages pg0;
+    if (part_start + 48 <= last_tile_tok) {  // (the early requests were for these four tiles)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pg0.p[j] = early_page[j];
+        pg0.off[j] = (part_start + 16 * j) & bs_mask;
+      }
+    } else {
+      pg0 = load_pages(part_start);
+    }
     issue_k(buf_a, pg0);
     issue_v(buf_a, pg0);
   }
