@@ -678,6 +678,7 @@ def _bench_trace(a) -> int:
     words = np.zeros(16384 * 8, dtype=np.uint64)
     _cabi.check(lib.pa_decode_trace_read(words.ctypes.data, words.nbytes), "pa_decode_trace_read")
     t = words.reshape(-1, 8).astype(np.float64)
+    xcd_of = (np.arange(len(t)) & 7)[t[:, 5] > 0]  # workgroup ids go round the eight XCDs
     t = t[t[:, 5] > 0]
     us = 0.01  # per tick
     ent, req, qry, first, last, end, steps, rows = [t[:, i] for i in range(8)]
@@ -702,6 +703,10 @@ def _bench_trace(a) -> int:
         "whole_workgroup": stat(end - ent),
         "slot_time_used": round(float((end - ent).sum() * us / (slots * span)), 3),
         "last_time_nine_tenths_of_the_slots_are_busy_us": round(tail_from, 1),
+        # per XCD: when its last workgroup ended, and the sum of its workgroups' times over its share of the slots
+        "xcd_end_us": [round(float((end[xcd_of == x].max() - start) * us), 1) for x in range(8)],
+        "xcd_busy_per_slot_us": [round(float((end - ent)[xcd_of == x].sum() * us / (slots / 8)), 1) for x in range(8)],
+        "xcd_per_step_us": [round(float((((last - first) / np.maximum(steps, 1))[(xcd_of == x) & (steps >= 16)]).mean() * us), 3) for x in range(8)],
         "per_step_us_by_live_rows": {str(r): round(float((((last - first) / steps)[(rows > r - 16) & (rows <= r) & (steps >= 16)]).mean() * us), 2)
                                      for r in (16, 32, 48, 64) if ((rows > r - 16) & (rows <= r) & (steps >= 16)).any()},
     }, ensure_ascii=False))

@@ -171,32 +171,35 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   } else {
     // The partition index varies slowest: in a ragged batch the partitions that only the longest
     // sequences reach (workgroups that exit at once for everybody else) come last.
-    const long long wid = blockIdx.x;
-    long long item;
+    // (32-bit unsigned arithmetic: the grid has fewer than 2^31 workgroups, and a 64-bit division by a run-time
+    // value is a hundred instructions in front of the workgroup's first request)
+    const uint32_t wid = blockIdx.x;
+    uint32_t item;
     if (PER_TOKEN && (a.flags & kFlagHeadsShareXcd)) {
       // Workgroup ids go round the eight XCDs: an XCD takes every eighth item with all its kv heads and row tiles one
       // after the other, so the 128-byte lines that hold the per-token scales of two neighbouring heads are
       // fetched into one L2 once (with the head fastest in the id every head sits on another XCD)
-      const int xcd = (int)(wid & 7);
-      const long long slot = wid >> 3;
-      const int unit = (int)(slot % (Hkv * RT));
-      h = unit % Hkv;
-      rt = unit / Hkv;
-      item = (slot / (Hkv * RT)) * 8 + xcd;
-      if (!(a.flags & kFlagSortedItems) && item >= (long long)a.num_seqs * ((P + span - 1) / span)) return;
+      const uint32_t xcd = wid & 7u;
+      const uint32_t slot = wid >> 3;
+      const uint32_t units = (uint32_t)(Hkv * RT);
+      const uint32_t unit = slot % units;
+      h = (int)(unit % (uint32_t)Hkv);
+      rt = (int)(unit / (uint32_t)Hkv);
+      item = (slot / units) * 8u + xcd;
+      if (!(a.flags & kFlagSortedItems) && item >= (uint32_t)a.num_seqs * (uint32_t)((P + span - 1) / span)) return;
     } else {
-      h = (int)(wid % Hkv);
-      rt = (int)((wid / Hkv) % RT);
-      item = wid / ((long long)Hkv * RT);
+      h = (int)(wid % (uint32_t)Hkv);
+      rt = (int)((wid / (uint32_t)Hkv) % (uint32_t)RT);
+      item = wid / (uint32_t)(Hkv * RT);
     }
     if (a.flags & kFlagSortedItems) {
       // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
-      if (item >= sload_i32(a.workspace + 2)) return;
-      b = sload_i32(a.workspace + kPlanHeaderWords + 2 * item);
-      part = sload_i32(a.workspace + kPlanHeaderWords + 2 * item + 1) * span;
+      if (item >= (uint32_t)sload_i32(a.workspace + 2)) return;
+      b = sload_i32(a.workspace + kPlanHeaderWords + 2 * (int64_t)item);
+      part = sload_i32(a.workspace + kPlanHeaderWords + 2 * (int64_t)item + 1) * span;
     } else {
-      b = (int)(item % a.num_seqs);
-      const int coarse = (int)(item / a.num_seqs);
+      b = (int)(item % (uint32_t)a.num_seqs);
+      const int coarse = (int)(item / (uint32_t)a.num_seqs);
       part = coarse * span;
       // (items go to the XCDs round robin: with a batch that is a multiple of eight every partition of a sequence
       // would sit on the same XCD, and a batch's one long sequence on one eighth of the GPU; each partition index

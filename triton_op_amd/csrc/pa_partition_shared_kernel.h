@@ -47,37 +47,39 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
   const int Hkv = a.num_kv_heads;
   const int G = a.group_size;
   const int Ge = a.q_len * G;
-  const long long wid = blockIdx.x;
+  // (32-bit unsigned arithmetic: the grid has fewer than 2^31 workgroups, and a 64-bit division by a run-time value
+  // is a hundred instructions in front of the workgroup's first request)
+  const uint32_t wid = blockIdx.x;
   int h;
-  long long item;
+  uint32_t item;
   if (a.flags & kFlagHeadsShareXcd) {
     // Workgroup ids go round the eight XCDs.  With the head fastest in the id, the kv heads of an item land on
     // eight different XCDs and each fetches the 128-byte lines that hold its own 64 bytes of per-token scales of a
     // page AND its neighbour's; here an XCD takes every eighth item with all its heads one after the other, so the
     // heads' scale lines (and nothing else: K and V are disjoint) meet in one L2.
-    const int xcd = (int)(wid & 7);
-    const long long slot = wid >> 3;
-    h = (int)(slot % Hkv);
-    item = (slot / Hkv) * 8 + xcd;
+    const uint32_t xcd = wid & 7u;
+    const uint32_t slot = wid >> 3;
+    h = (int)(slot % (uint32_t)Hkv);
+    item = (slot / (uint32_t)Hkv) * 8u + xcd;
   } else {
-    h = (int)(wid % Hkv);
-    item = wid / Hkv;
+    h = (int)(wid % (uint32_t)Hkv);
+    item = wid / (uint32_t)Hkv;
   }
   int b, part;
   if (a.flags & kFlagSortedItems) {
     // the planning kernel has listed the live (sequence, partition) items, longest last partitions first
     // (the number of listed items and this item's record are requested together: the list area is sized for every
     // (sequence, partition) pair, and the grid's padding items read the last record)
-    const long long pairs = (long long)a.num_seqs * a.max_num_partitions;
-    const long long rec = item < pairs ? item : pairs - 1;
+    const uint32_t pairs = (uint32_t)a.num_seqs * (uint32_t)a.max_num_partitions;
+    const int64_t rec = item < pairs ? item : pairs - 1;
     const int listed = sload_i32(a.workspace + 2);
     b = sload_i32(a.workspace + kPlanHeaderWords + 2 * rec);
     part = sload_i32(a.workspace + kPlanHeaderWords + 2 * rec + 1);
-    if (item >= listed) return;
+    if (item >= (uint32_t)listed) return;
   } else {
-    if (item >= (long long)a.num_seqs * a.max_num_partitions) return;  // (the grid is whole groups of eight items)
-    b = (int)(item % a.num_seqs);
-    part = (int)(item / a.num_seqs);
+    if (item >= (uint32_t)a.num_seqs * (uint32_t)a.max_num_partitions) return;  // (the grid is whole groups of eight items)
+    b = (int)(item % (uint32_t)a.num_seqs);
+    part = (int)(item / (uint32_t)a.num_seqs);
     // (items go to the XCDs round robin: with a batch that is a multiple of eight every partition of a sequence
     // would sit on the same XCD, and a batch's one long sequence on one eighth of the GPU; each partition index
     // therefore starts the batch one sequence further on)
