@@ -696,7 +696,19 @@ def _random_case(seed):
     return kw, ps, alibi
 
 
-@pytest.mark.parametrize("seed", range(48))
+def _sweep_seeds():
+    """48 seeds in every run; PA_SWEEP_SEEDS=lo:hi (e.g. 48:14048) runs that range instead -- a soak for whoever
+    changes the kernels (about a minute per 2000 seeds on the GPU)."""
+    import os
+
+    span = os.environ.get("PA_SWEEP_SEEDS", "")
+    if span:
+        lo, _, hi = span.partition(":")
+        return range(int(lo), int(hi))
+    return range(48)
+
+
+@pytest.mark.parametrize("seed", _sweep_seeds())
 def test_seeded_random_sweep(cuda, seed):
     """Random shapes, layouts, scale modes, partition sizes and ALiBi: the HIP path against the oracle end to
     end and stage by stage."""
