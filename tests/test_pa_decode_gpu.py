@@ -962,3 +962,86 @@ def test_output_only_flag(cuda, pa_lib, name, partition_size, with_sinks):
         if finished_by_stage_1 and ctx > 0:
             assert torch.all(view(out)[b, :, ql:] == 7.0), f"padding rows of sequence {b} were written"
             assert torch.all(p.exp_sums[b] == -3.0), f"partition-buffer entries of sequence {b} were written"
+
+
+def _random_case_wide(seed):
+    """A second seeded draw: larger batches (launches of several rounds: sorted dispatch, grids padded to whole groups
+    of eight items, the item list's reuse), attention sinks, an FP8 query with per-row or per-tensor scale, the
+    caller's total-token statistic and PA_DECODE_FLAG_OUTPUT_ONLY, in any combination."""
+    gen = torch.Generator().manual_seed(777000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=gen))]
+
+    kv_dtype = pick(["fp8", "fp8", "fp8", "bf16"])
+    q_len = pick([1, 2, 4])
+    group = pick([g for g in (1, 4, 8, 16) if g * q_len <= 64])
+    hkv = pick([1, 2, 8])
+    batch = pick([3, 17, 40, 64])
+    shape = pick(["short", "mixed", "skewed"])
+    hi = {"short": 300, "mixed": 1500, "skewed": 200}[shape]
+    ctx = torch.randint(q_len, hi + 1, (batch,), generator=gen, dtype=torch.int32)
+    if shape == "skewed":
+        ctx[int(torch.randint(0, batch, (1,), generator=gen))] = pick([3000, 6000])
+    kw = dict(batch=batch, num_q_heads=group * hkv, num_kv_heads=hkv, context_lens=ctx, q_len=q_len,
+              block_size=pick([16, 16, 64]), kv_dtype=kv_dtype, seed=seed,
+              scale_mode="none" if kv_dtype == "bf16" else pick(["tensor", "token"]), transposed_v=pick([False, True]))
+    if q_len > 1 and pick([False, True]):
+        kw["q_lens"] = torch.randint(1, q_len + 1, (batch,), generator=gen, dtype=torch.int32)
+    opts = dict(partition_size=pick([256, 256, 512, None]), sinks=pick([False, True]),
+                fp8_query=pick(["no", "no", "row", "tensor"]), output_only=pick([False, True]),
+                total=pick([False, True]), alibi=pick([False, False, True]))
+    return kw, opts
+
+
+def _wide_seeds():
+    import os
+
+    span = os.environ.get("PA_SWEEP_SEEDS_WIDE", "")
+    if span:
+        lo, _, hi = span.partition(":")
+        return range(int(lo), int(hi))
+    return range(32)
+
+
+@pytest.mark.parametrize("seed", _wide_seeds())
+def test_seeded_random_sweep_wide(cuda, seed):
+    """The features the first sweep does not draw, against the oracle end to end (real query rows only when the call
+    is made with output_only); PA_SWEEP_SEEDS_WIDE=lo:hi runs another range of the draw."""
+    import triton_op_amd as T
+    from triton_op_amd import kv_layout as L
+
+    kw, o = _random_case_wide(seed)
+    print(f"seed={seed} {o} " + " ".join(f"{k}={v.tolist() if torch.is_tensor(v) else v}" for k, v in kw.items()), flush=True)
+    wl = _make(**kw)
+    g = wl.to(cuda)
+    rows = wl.query.shape[1]
+    query, qscale = wl.query, None
+    if o["fp8_query"] == "row":
+        query, qscale = L.pertoken_quant(wl.query.float())
+    elif o["fp8_query"] == "tensor":
+        qscale = torch.tensor(max(float(wl.query.float().abs().max()), 1e-6) / 448.0)
+        query = (wl.query.float() / qscale).to(torch.float8_e4m3fn)
+    sinks = torch.linspace(-2.0, 2.0, rows, dtype=torch.float32) if o["sinks"] else None
+    slopes = torch.linspace(0.02, 0.4, rows if seed % 2 else wl.num_q_heads, dtype=torch.float32) if o["alibi"] else None
+    out = torch.full_like(g.query, float("nan"))
+    dev = lambda t: None if t is None else t.to(cuda)
+    T.paged_attention_decode(
+        out, dev(query), g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale, g.q_len,
+        g.max_context_len, torch.bfloat16, dev(qscale), g.key_scale, g.value_scale, alibi_slopes=dev(slopes),
+        partition_size=o["partition_size"], query_lens=g.q_lens, sinks=dev(sinks), output_only=o["output_only"],
+        total_context_tokens=int(wl.context_lens.sum()) if o["total"] else 0)
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode_oracle(
+        query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
+        wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, slopes, None, query_scale=qscale,
+        q_max=wl.q_len, sinks=sinks)
+    got = out.float().cpu()
+    hkv, q_max = wl.key_cache.shape[1], wl.q_len
+    view = lambda t: t.view(t.shape[0], hkv, q_max, -1, t.shape[-1])
+    qls = wl.q_lens.tolist() if wl.q_lens is not None else [q_max] * wl.batch
+    for b, ql in enumerate(qls):  # the real query rows (the others are unspecified under output_only)
+        torch.testing.assert_close(view(got)[b, :, :ql], view(ref.float())[b, :, :ql], atol=ATOL, rtol=RTOL)
+    if not o["output_only"]:
+        assert not torch.isnan(got).any()
+        torch.testing.assert_close(got, ref.float(), atol=ATOL, rtol=RTOL)
