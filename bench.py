@@ -5,7 +5,7 @@
                                                                      256-token partitions, c3, c4 and c5 in `configs`
     python bench.py --workload c1|c2|c3|c4|c5 [--partition-size N]   one configuration
     python bench.py --workload ref:B,Hq,Hkv,bs,qlen[,transv][,ctx=N]  one row of the reference harness's sweep
-    python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1]
+    python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1,hd=64|128|256]
                                [,lens=c5[,qlens=c5|N][,pick=one|rest]]   c5's draw of context lengths (and of new tokens per sequence)
     python bench.py --workload probe_gather                          read-only probe of c2's page-gather pattern
     python bench.py --workload probe_gather:c5                       ... of another workload's (plain order, four-wave workgroups)
@@ -139,7 +139,8 @@ def _make_custom_workload(spec, device, seed):
     q, ctx, bs = int(kv.get("q", 1)), int(kv.get("ctx", 4096)), int(kv.get("bs", 16))
     scale, kvd, qd = kv.get("scale", "tensor"), kv.get("kv", "fp8"), kv.get("qdtype", "bf16")
     transv = kv.get("transv", "0") == "1"
-    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv", "lens", "qlens", "pick"}
+    hd = int(kv.get("hd", 128))  # head size: 128 on the tuned kernels, 64 / 256 on the generic ones
+    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv", "lens", "qlens", "pick", "hd"}
     if unknown:
         raise ValueError(f"custom: unknown keys {sorted(unknown)}")
     ctx_lens, q_lens, tag = torch.full((b,), ctx, dtype=torch.int32), None, f"ctx{ctx}"
@@ -163,8 +164,8 @@ def _make_custom_workload(spec, device, seed):
     elif "lens" in kv or "qlens" in kv:
         raise ValueError("custom: lens=c5 is the only length distribution on offer; qlens needs it")
     wl = W.make_decode_workload(
-        name=f"custom_b{b}_h{hq}x{hkv}_bs{bs}_q{q}_{tag}_{kvd}_{scale}_{qd}q{'_transv' if transv else ''}", seed=seed,
-        batch=b, num_q_heads=hq, num_kv_heads=hkv, block_size=bs,
+        name=f"custom_b{b}_h{hq}x{hkv}_bs{bs}_q{q}_{tag}_{kvd}_{scale}_{qd}q{'_transv' if transv else ''}{'' if hd == 128 else f'_hd{hd}'}",
+        seed=seed, batch=b, num_q_heads=hq, num_kv_heads=hkv, block_size=bs, head_size=hd,
         context_lens=ctx_lens, q_len=q, q_lens=q_lens, kv_dtype=kvd,
         scale_mode="none" if kvd == "bf16" else scale, device=device, transposed_v=transv)
     if qd == "fp8":

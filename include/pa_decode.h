@@ -123,7 +123,8 @@ typedef struct PaDecodeArgs {
   int32_t num_kv_heads;
   int32_t group_size;          /* G */
   int32_t q_len;               /* q (the maximum over the batch when q_lens is given) */
-  int32_t head_size;           /* D, 128 */
+  int32_t head_size;           /* D: 128 (the tuned kernels), or 64 / 256 (generic kernels: same results, about half the
+                                  rate); anything else is PA_ERR_UNSUPPORTED */
   int32_t block_size;          /* 16, 64 or 1024 */
   int32_t max_num_partitions;  /* P: partition axis length of the three buffers; P * partition_size must cover the
                                   longest context_len (the caller's max_sequence_length sizes it): tokens beyond it

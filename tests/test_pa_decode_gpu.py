@@ -643,7 +643,7 @@ def test_c_abi_rejects_bad_arguments(cuda, pa_lib):
                          wl.softmax_scale, 1, 300, torch.bfloat16, None, wl.key_scale, wl.value_scale)
     a = plan.args
     assert pa_lib.pa_decode(None, None) == -1
-    for field, bad, code in (("struct_size", 8, -2), ("head_size", 64, -3), ("block_size", 32, -3),
+    for field, bad, code in (("struct_size", 8, -2), ("head_size", 96, -3), ("block_size", 32, -3),
                              ("partition_size", 100, -4), ("key_cache", None, -1), ("num_seqs", 0, -4),
                              ("stride_k_b", 8, -4)):
         good = getattr(a, field)
@@ -1044,4 +1044,88 @@ def test_seeded_random_sweep_wide(cuda, seed):
         torch.testing.assert_close(view(got)[b, :, :ql], view(ref.float())[b, :, :ql], atol=ATOL, rtol=RTOL)
     if not o["output_only"]:
         assert not torch.isnan(got).any()
+        torch.testing.assert_close(got, ref.float(), atol=ATOL, rtol=RTOL)
+
+
+GENERIC_HEAD_CASES = ["fp8_g8", "fp8_g8_boundaries", "fp8_g5_q2", "fp8_g16_q4", "fp8_token_ragged", "fp8_token_g8_q1",
+                      "bf16_g8", "bf16_g16_q4", "fp8_bs1024_q2", "fp8_bs64", "fp8_transV_bs16", "fp8_transV_bs1024",
+                      "fp8_token_transV_bs64_g8_q3", "bf16_ragged_g16_q4", "bf16_transV_bs64",
+                      "fp8_ragged_two_waves_per_tile"]
+
+
+@pytest.mark.parametrize("head_size", [64, 256])
+@pytest.mark.parametrize("name", GENERIC_HEAD_CASES)
+@pytest.mark.parametrize("partition_size", [256, 1024])
+def test_head_sizes_64_and_256(cuda, head_size, name, partition_size):
+    """Head sizes other than 128 run on the generic kernels (plain f32 arithmetic): the same cases as the tuned
+    kernels', stage by stage and end to end against the oracle."""
+    import triton_op_amd as T
+
+    wl = _make(**CASES[name], head_size=head_size)
+    g = wl.to(cuda)
+    info = T.plan_decode(torch.empty_like(g.query), g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables,
+                         g.softmax_scale, g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                         partition_size=partition_size, query_lens=g.q_lens).launch_info()
+    assert info.startswith(f"pa_partition_generic_kernel<head size {head_size}"), info
+    out, res = _run(wl, cuda, partition_size=partition_size)
+    assert not torch.isnan(out.float()).any()
+    _check_stages(wl, res, partition_size)
+    torch.testing.assert_close(out.float(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("head_size", [64, 256])
+@pytest.mark.parametrize("feature", ["alibi_rows", "alibi_heads", "sinks", "fp8_query_rows", "fp8_query_tensor",
+                                     "output_only", "noalloc", "stale_nan"])
+def test_head_sizes_64_and_256_options(cuda, head_size, feature):
+    """... and the operator's options on those head sizes."""
+    import triton_op_amd as T
+    from triton_op_amd import kv_layout as L
+
+    wl = _make(batch=4, num_q_heads=32, num_kv_heads=2, context_lens=_ctx(700, 33, 300, 5), q_len=2,
+               q_lens=_ctx(2, 1, 2, 2), scale_mode="token", head_size=head_size)
+    g = wl.to(cuda)
+    rows = wl.query.shape[1]
+    query, qscale, slopes, sinks = wl.query, None, None, None
+    if feature == "alibi_rows":
+        slopes = torch.linspace(0.02, 0.4, rows, dtype=torch.float32)
+    if feature == "alibi_heads":
+        slopes = torch.linspace(0.02, 0.4, wl.num_q_heads, dtype=torch.float32)
+    if feature == "sinks":
+        sinks = torch.linspace(-2.0, 3.0, rows, dtype=torch.float32)
+    if feature == "fp8_query_rows":
+        query, qscale = L.pertoken_quant(wl.query.float())
+    if feature == "fp8_query_tensor":
+        qscale = torch.tensor(float(wl.query.float().abs().max()) / 448.0)
+        query = (wl.query.float() / qscale).to(torch.float8_e4m3fn)
+    if feature == "stale_nan":  # cache bytes past every sequence's end decode to NaN: they must never reach a result
+        kc, vc = g.key_cache.view(torch.uint8).clone(), g.value_cache.view(torch.uint8).clone()
+        bs = wl.key_cache.shape[-2]
+        for b in range(wl.batch):
+            ctx = int(wl.context_lens[b])
+            blk = int(wl.block_tables[b, (ctx - 1) // bs])
+            kc[blk, :, :, ctx % bs if ctx % bs else bs:, :] = 0x7f
+            vc[blk, :, :, ctx % bs if ctx % bs else bs:] = 0x7f
+        g = type(g)(**{**g.__dict__, "key_cache": kc.view(g.key_cache.dtype), "value_cache": vc.view(g.value_cache.dtype)})
+    dev = lambda t: None if t is None else t.to(cuda)
+    out = torch.full_like(g.query, 7.0)
+    plan = T.plan_decode(out, dev(query), g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                         g.q_len, g.max_context_len, torch.bfloat16, dev(qscale), g.key_scale, g.value_scale,
+                         alibi_slopes=dev(slopes), partition_size=256, query_lens=g.q_lens, sinks=dev(sinks),
+                         output_only=feature == "output_only")
+    if feature == "noalloc":
+        plan.run_noalloc()
+    else:
+        plan.run()
+    torch.cuda.synchronize()
+    ref = O.paged_attention_decode_oracle(
+        query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale, wl.q_lens,
+        wl.key_scale, wl.value_scale, slopes, None, query_scale=qscale, q_max=wl.q_len, sinks=sinks)
+    got = out.float().cpu()
+    hkv, q_max = wl.key_cache.shape[1], wl.q_len
+    view = lambda t: t.view(t.shape[0], hkv, q_max, -1, t.shape[-1])
+    for b, ql in enumerate(wl.q_lens.tolist()):
+        torch.testing.assert_close(view(got)[b, :, :ql], view(ref.float())[b, :, :ql], atol=ATOL, rtol=RTOL)
+        if feature == "output_only":
+            assert torch.all(view(got)[b, :, ql:] == 7.0)
+    if feature != "output_only":
         torch.testing.assert_close(got, ref.float(), atol=ATOL, rtol=RTOL)

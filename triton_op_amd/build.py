@@ -17,7 +17,7 @@ SOURCES = [os.path.join(HERE, "csrc", "pa_decode.hip"), os.path.join(HERE, "csrc
 HEADERS = [os.path.join(HERE, "..", "include", "pa_decode.h")] + [
     os.path.join(HERE, "csrc", h)
     for h in ("pa_common.h", "pa_launch.h", "pa_partition_kernel.h", "pa_partition_shared_kernel.h", "pa_plan_kernel.h",
-              "pa_reduce_kernel.h")]
+              "pa_reduce_kernel.h", "pa_generic_kernel.h")]
 LIB_PATH = os.path.join(HERE, "libpa_decode.so")
 
 HIPCC_FLAGS = [

@@ -20,6 +20,7 @@
 #include "pa_launch.h"
 #include "pa_partition_kernel.h"
 #include "pa_partition_shared_kernel.h"
+#include "pa_generic_kernel.h"
 #include "pa_plan_kernel.h"
 #include "pa_reduce_kernel.h"
 
@@ -60,7 +61,7 @@ int check_common(const PaDecodeArgs* a) {
   if (a->partition_size <= 0 || a->partition_size % 256) return PA_ERR_BAD_SHAPE;
   if (a->flags & ~(PA_DECODE_FLAG_REUSE_ITEM_LIST | PA_DECODE_FLAG_OUTPUT_ONLY)) return PA_ERR_BAD_SHAPE;
   if (a->workspace ? a->workspace_bytes < PA_DECODE_WORKSPACE_BYTES : a->workspace_bytes != 0) return PA_ERR_BAD_SHAPE;
-  if (a->head_size != kHeadSize) return PA_ERR_UNSUPPORTED;
+  if (a->head_size != kHeadSize && a->head_size != 64 && a->head_size != 256) return PA_ERR_UNSUPPORTED;
   if (a->q_len * a->group_size > 64) return PA_ERR_UNSUPPORTED;  // the reference's limit
   return PA_OK;
 }
@@ -282,6 +283,40 @@ int launch_partition_shared(const PaDecodeArgs& a, const LaunchChoice& c, hipStr
     return pa_launch(pa_partition_shared_kernel<true, BS16, 3, 3>, dim3((unsigned)c.blocks), dim3(256), (unsigned)pad, stream, k);
   else
     return pa_launch(pa_partition_shared_kernel<false, BS16, 2, 4>, dim3((unsigned)c.blocks), dim3(256), (unsigned)pad, stream, k);
+}
+
+int check_reduce(const PaDecodeArgs* a);
+
+// Head sizes other than 128 (64 and 256) run on the two generic kernels (pa_generic_kernel.h): plain order, one wave
+// per (sequence, partition, kv head, 16-row tile), and a merge that always runs.
+bool generic_head_size(const PaDecodeArgs& a) { return a.head_size != kHeadSize; }
+
+long long generic_partition_blocks(const PaDecodeArgs& a) {
+  return (long long)a.num_seqs * a.max_num_partitions * a.num_kv_heads * ((a.q_len * a.group_size + 15) / 16);
+}
+
+int launch_partition_generic(const PaDecodeArgs& a, hipStream_t stream) {
+  const long long blocks = generic_partition_blocks(a);
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  PaDecodeArgs k = a;
+  k.flags = (a.flags & PA_DECODE_FLAG_OUTPUT_ONLY) ? kFlagOutputOnly : 0;
+  const dim3 grid((unsigned)blocks), block(64);
+  const bool fp8 = a.kv_dtype == PA_DTYPE_FP8_E4M3FN;
+  if (a.head_size == 64)
+    return fp8 ? pa_launch(pa_partition_generic_kernel<64, true>, grid, block, 0, stream, k)
+               : pa_launch(pa_partition_generic_kernel<64, false>, grid, block, 0, stream, k);
+  return fp8 ? pa_launch(pa_partition_generic_kernel<256, true>, grid, block, 0, stream, k)
+             : pa_launch(pa_partition_generic_kernel<256, false>, grid, block, 0, stream, k);
+}
+
+int launch_reduce_generic(const PaDecodeArgs* a, void* hip_stream) {
+  const int rc = check_reduce(a);
+  if (rc) return rc;
+  const long long blocks = (long long)a->num_seqs * a->num_kv_heads * a->q_len * a->group_size;
+  if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+  if (a->head_size == 64) return pa_launch(pa_reduce_generic_kernel<64>, dim3((unsigned)blocks), dim3(64), 0, stream, *a);
+  return pa_launch(pa_reduce_generic_kernel<256>, dim3((unsigned)blocks), dim3(64), 0, stream, *a);
 }
 
 // stage 1 as chosen: the planning kernel when the items are to be sorted, then the partition kernel
@@ -539,12 +574,14 @@ int pa_decode_select_partition_size_stats(int32_t num_seqs_given, int32_t num_kv
 int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
   const int rc = check_partition(a);
   if (rc) return rc;
+  if (generic_head_size(*a)) return launch_partition_generic(*a, reinterpret_cast<hipStream_t>(hip_stream));
   return launch_partition(*a, choose_launch(*a), reinterpret_cast<hipStream_t>(hip_stream));
 }
 
 int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
   // PA_DECODE_FLAG_OUTPUT_ONLY: stage 1 ran with the same flag and left no entries for the sequences it finished
   // itself; stage 2 passes over them, as it does inside pa_decode
+  if (a && a->struct_size == sizeof(PaDecodeArgs) && generic_head_size(*a)) return launch_reduce_generic(a, hip_stream);
   const bool lean = a && a->struct_size == sizeof(PaDecodeArgs) && (a->flags & PA_DECODE_FLAG_OUTPUT_ONLY);
   if (lean && a->max_num_partitions == 1 && !a->sinks) {
     const int rc = check_reduce(a);
@@ -558,6 +595,10 @@ int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
   if (rc) return rc;
   rc = check_reduce(a);  // before anything is launched
   if (rc) return rc;
+  if (generic_head_size(*a)) {
+    rc = launch_partition_generic(*a, reinterpret_cast<hipStream_t>(hip_stream));
+    return rc ? rc : launch_reduce_generic(a, hip_stream);
+  }
   const LaunchChoice c = choose_launch(*a);
   rc = launch_partition(*a, c, reinterpret_cast<hipStream_t>(hip_stream));
   if (rc) return rc;
@@ -571,6 +612,11 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
   const int rc = check_partition(a);
   if (rc) return rc;
   if (!text || text_bytes <= 0) return PA_ERR_NULL_POINTER;
+  if (generic_head_size(*a)) {
+    snprintf(text, (size_t)text_bytes, "pa_partition_generic_kernel<head size %d, %s> x %lld", a->head_size,
+             a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? "fp8" : "bf16", generic_partition_blocks(*a));
+    return PA_OK;
+  }
   const LaunchChoice c = choose_launch(*a);
   const char* cache = !c.fp8 ? "bf16" : (c.per_token ? "fp8 per-token" : "fp8");
   const char* placed = c.heads_share_xcd ? ", an item's heads on one XCD" : "";
@@ -643,9 +689,9 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
   const long long limit = (long long)PA_DECODE_NOALLOC_SCRATCH_BYTES;
   long long rows = 0, tmp_bytes = 0;
   if (__builtin_mul_overflow((long long)a->num_seqs * a->num_kv_heads, (long long)a->max_num_partitions * ge, &rows) ||
-      __builtin_mul_overflow(rows, 2LL * kHeadSize, &tmp_bytes) || tmp_bytes > limit)
+      __builtin_mul_overflow(rows, 2LL * a->head_size, &tmp_bytes) || tmp_bytes > limit)
     return PA_ERR_SCRATCH_TOO_SMALL;
-  // (rows * 256 <= 64 MiB bounds num_seqs * max_num_partitions by 2^18: the workspace size cannot overflow either)
+  // (rows * 128 <= 64 MiB bounds num_seqs * max_num_partitions by 2^19: the workspace size cannot overflow either)
   const long long ws_bytes = full_workspace_bytes(a->num_seqs, a->max_num_partitions);
   if (ws_bytes > limit) return PA_ERR_SCRATCH_TOO_SMALL;
   const long long off_ml = round256(ws_bytes);
@@ -663,8 +709,8 @@ int pa_decode_noalloc(const PaDecodeArgs* a, void* hip_stream) {
   k.stride_es_p = ge;
   k.stride_es_h = ge * a->max_num_partitions;
   k.stride_es_s = k.stride_es_h * a->num_kv_heads;
-  k.stride_tmp_g = kHeadSize;
-  k.stride_tmp_p = ge * kHeadSize;
+  k.stride_tmp_g = a->head_size;
+  k.stride_tmp_p = ge * a->head_size;
   k.stride_tmp_h = k.stride_tmp_p * a->max_num_partitions;
   k.stride_tmp_s = k.stride_tmp_h * a->num_kv_heads;
   // the array keeps the last call's contents (a call that was cut short may have left its counters non-zero, and

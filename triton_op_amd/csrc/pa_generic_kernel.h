@@ -1,0 +1,286 @@
+// pa_partition_generic_kernel / pa_reduce_generic_kernel: both stages for head sizes other than 128.
+#ifndef PA_GENERIC_KERNEL_H_
+#define PA_GENERIC_KERNEL_H_
+
+#include "pa_common.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// The reference's kernels take any power-of-two head size (pa_decode_triton_gluon_fp8.py:514-1002 pads it to
+// HEAD_SIZE_POW2); its sweep, its published numbers and the tuned kernels of this library are all at 128.  Head
+// sizes 64 and 256 run on the two kernels of this file: every layout, dtype, scale mode and option of the operator,
+// on bf16 MFMAs without a software pipeline -- the same results, not the same speed.
+//
+// Stage 1: one wave per (sequence, partition, kv head, 16-row query tile).  A 64-token step is four 16-token
+// tiles.  v_mfma_f32_16x16x16_bf16 holds, in lane l (li = l % 16, kg = l / 16), four consecutive reduction indices
+// 4 kg .. 4 kg + 3 of row / column li of its operands and rows 4 kg .. 4 kg + 3 of column li of its result, so:
+//   S^T[token, row] = K Q^T:  A = 4 head dims of token li (4 or 8 bytes of the cache, converted to bf16),
+//                             B = the same 4 head dims of query row li; the result holds 4 tokens of row li;
+//   O^T[dim, row]   = V^T P:  A = 4 tokens of head dim li of a 16-dim block, B = P of those 4 tokens for row li --
+//                             exactly what the lane holds of S^T, so P never moves between lanes.
+// Row maximum and sum: 16 values in the lane, then the four lanes of a row (quad_row_max / quad_row_sum).
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) short bf16x4_bits;
+
+// four consecutive cache elements starting at p as bf16 (FP8 values are exact in bf16)
+template <bool FP8>
+__device__ __forceinline__ bf16x4_bits load_cache4(const char* p) {
+  union {
+    bf16x4_bits v;
+    uint32_t u[2];
+  } r;
+  if constexpr (FP8) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+    r.u[0] = fp8x2_to_bf16x2(w, false);
+    r.u[1] = fp8x2_to_bf16x2(w, true);
+  } else {
+    const u32x2 w = *reinterpret_cast<const u32x2*>(p);
+    r.u[0] = w[0];
+    r.u[1] = w[1];
+  }
+  return r.v;
+}
+
+// (there is no prefetch: the waves of a SIMD hide each other's load latency, so the registers are capped for four
+// waves per SIMD, two with the 64 accumulator registers of head size 256)
+template <int D, bool FP8>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(D > 128 ? 2 : 4, D > 128 ? 2 : 4)))
+void pa_partition_generic_kernel(const PaDecodeArgs a) {
+  constexpr int X = FP8 ? 16 : 8;  // cache elements per 16 bytes
+  constexpr int ESZ = FP8 ? 1 : 2;
+  constexpr int DB = D / 16;       // 16-dim blocks of the head
+  static_assert(D % 16 == 0, "the head is cut into 16-dim blocks");
+
+  const int lane = threadIdx.x;
+  const int li = lane & 15, kg = lane >> 4;
+  const int Hkv = a.num_kv_heads;
+  const int G = a.group_size;
+  const int Ge = a.q_len * G;
+  const int RT = (Ge + 15) / 16;
+  const uint32_t wid = blockIdx.x;
+  const int h = (int)(wid % (uint32_t)Hkv);
+  const int rt = (int)((wid / (uint32_t)Hkv) % (uint32_t)RT);
+  const uint32_t item = wid / (uint32_t)(Hkv * RT);
+  const int b = (int)(item % (uint32_t)a.num_seqs);
+  const int part = (int)(item / (uint32_t)a.num_seqs);
+  const int row0 = 16 * rt;
+
+  const int ctx = sload_i32(a.context_lens + b);
+  const int wg_start = part * a.partition_size;
+  if (wg_start >= ctx && !(ctx <= 0 && part == 0)) return;  // (an empty sequence keeps its first partition: zeros)
+  const int wg_end = min(wg_start + a.partition_size, ctx);
+  const int qb = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
+  const int rows_valid = qb * G;
+  const bool output_only = a.flags & kFlagOutputOnly;
+
+  const int64_t es_off = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)part * a.stride_es_p;
+  char* tmp = (char*)a.tmp_output +
+              ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h + (int64_t)part * a.stride_tmp_p) * 2;
+
+  // ---- this lane's query row: its B operands (4 head dims per 16-dim block), its scale, its mask ------------------
+  const int row = row0 + li;
+  const bool row_ok = row < rows_valid;
+  const int t_row = row / G;
+  const int limit = row_ok ? ctx - (qb - 1 - t_row) : 0;  // number of visible keys (causal over the new tokens)
+  float k_tensor_scale = 1.f, v_tensor_scale = 1.f;
+  if (a.kv_quant_mode == PA_QUANT_PER_TENSOR) {
+    k_tensor_scale = sload_f32(a.key_scale);
+    v_tensor_scale = sload_f32(a.value_scale);
+  }
+  const bool per_token = a.kv_quant_mode == PA_QUANT_PER_TOKEN;
+  float rscale = a.softmax_scale * k_tensor_scale * kLog2e;  // logits in the log2 domain
+  if (a.query_quant_mode == PA_QUANT_PER_TENSOR) rscale *= sload_f32(a.query_scale);
+  if (a.query_quant_mode == PA_QUANT_PER_TOKEN && row_ok)
+    rscale *= a.query_scale[(int64_t)b * a.stride_qscale_s + h * Ge + row];
+  float slope2 = 0.f;
+  if (a.alibi_slopes && row_ok)
+    slope2 = a.alibi_slopes[a.alibi_slopes_len == Hkv * Ge ? h * Ge + row : h * G + (row - t_row * G)] * kLog2e;
+  bf16x4_bits qreg[DB];
+  {
+    const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (row_ok ? row : 0)) * a.stride_q_h + 4 * kg;
+#pragma unroll
+    for (int c = 0; c < DB; ++c) {
+      if (a.query_dtype == PA_DTYPE_BF16)
+        qreg[c] = load_cache4<false>((const char*)a.query + (e0 + 16 * c) * 2);
+      else
+        qreg[c] = load_cache4<true>((const char*)a.query + (e0 + 16 * c));
+      if (!row_ok) qreg[c] = bf16x4_bits{0, 0, 0, 0};
+    }
+  }
+
+  const int log2_bs = 31 - __builtin_clz(a.block_size);
+  const int bs_mask = a.block_size - 1;
+  const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
+  const char* kbase = (const char*)a.key_cache + (int64_t)h * a.stride_k_h * ESZ;
+  const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h * ESZ;
+  const int last_tile_tok = (max(wg_end, 1) - 1) & ~15;
+
+  float m_run = -INFINITY, l_run = 0.f;  // of row li (the same in the row's four lanes)
+  f32x4 acc[DB];                         // O^T: head dims 16 db + 4 kg .. + 3 of row li
+#pragma unroll
+  for (int db = 0; db < DB; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int tok0 = wg_start; tok0 < wg_end; tok0 += kStepTokens) {
+    // ---- pages of the step's four tiles (tiles past the last live one repeat it) ----------------------------------
+    int page[4], off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int t = tok0 + 16 * j;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      page[j] = sload_i32(bt + (t >> log2_bs));
+      off[j] = t & bs_mask;
+    }
+    // ---- S^T = K Q^T --------------------------------------------------------------------------------------------------
+    f32x4 s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const char* kt = kbase + (int64_t)page[j] * a.stride_k_b * ESZ;
+#pragma unroll
+      for (int c = 0; c < DB; ++c) {
+        const int d = 16 * c + 4 * kg;  // this lane's four head dims: inside one chunk of X dims
+        const bf16x4_bits ka =
+            load_cache4<FP8>(kt + ((int64_t)(d / X) * a.stride_k_c + (off[j] + li) * X + d % X) * ESZ);
+        s[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka, qreg[c], s[j], 0, 0, 0);
+      }
+    }
+    // ---- scales, ALiBi, mask; row maximum ---------------------------------------------------------------------------
+    f32x4 vs[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f32x4 ks = {1.f, 1.f, 1.f, 1.f};
+      vs[j] = f32x4{1.f, 1.f, 1.f, 1.f};
+      if (per_token) {
+        const int64_t so = (int64_t)page[j] * a.stride_kvscale_b + (int64_t)h * a.stride_kvscale_h + off[j] + 4 * kg;
+        ks = *reinterpret_cast<const f32x4*>(a.key_scale + so);
+        vs[j] = *reinterpret_cast<const f32x4*>(a.value_scale + so);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int col = tok0 + 16 * j + 4 * kg + r;
+        float x = s[j][r] * ks[r] * rscale + slope2 * (float)(col - ctx + 1);
+        x = col < limit ? x : -INFINITY;  // (a select: stale cache bytes may have made the logit a NaN)
+        s[j][r] = x;
+        mx = fmaxf(mx, x);
+      }
+    }
+    mx = quad_row_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);  // exp2(-inf) = 0 while the row has seen no key
+    m_run = m_new;
+    float psum = 0.f;
+    bf16x4_bits pb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float p[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        p[r] = fast_exp2(s[j][r] - m_safe);
+        psum += p[r];
+        p[r] *= vs[j][r];
+      }
+      union {
+        bf16x4_bits v;
+        uint32_t u[2];
+      } pk;
+      pk.u[0] = pack_bf16x2(p[0], p[1]);
+      pk.u[1] = pack_bf16x2(p[2], p[3]);
+      pb[j] = pk.v;
+    }
+    l_run = l_run * alpha + quad_row_sum(psum);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[db] *= alpha;
+    // ---- O^T += V^T P -----------------------------------------------------------------------------------------------
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t4 = tok0 + 16 * j + 4 * kg;  // this lane's four tokens of the tile
+      const int o4 = off[j] + 4 * kg;
+      const char* vt = vbase + (int64_t)page[j] * a.stride_v_b * ESZ;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = 16 * db + li;
+        const int64_t e = a.v_transposed ? (int64_t)(o4 / X) * a.stride_v_2 + (int64_t)d * X + o4 % X
+                                         : (int64_t)d * a.stride_v_2 + o4;
+        union {
+          bf16x4_bits v;
+          uint16_t h4[4];
+        } va;
+        va.v = load_cache4<FP8>(vt + e * ESZ);
+        // stale bytes past the context may decode to NaN, and 0 * NaN is NaN: those tokens' V is zero
+#pragma unroll
+        for (int r = 0; r < 4; ++r) va.h4[r] = t4 + r < ctx ? va.h4[r] : (uint16_t)0;
+        acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va.v, pb[j], acc[db], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- the partition's result: (max, sum, O / sum) of row li ---------------------------------------------------------
+  const int rows_live = output_only ? rows_valid : Ge;
+  if (row < rows_live) {
+    const float inv = l_run > 0.f ? v_tensor_scale / l_run : 0.f;
+    if (kg == 0) {
+      a.max_logits[es_off + row] = m_run * (1.0f / kLog2e);
+      a.exp_sums[es_off + row] = l_run;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      u32x2 pk;
+      pk[0] = pack_bf16x2(acc[db][0] * inv, acc[db][1] * inv);
+      pk[1] = pack_bf16x2(acc[db][2] * inv, acc[db][3] * inv);
+      *reinterpret_cast<u32x2*>(tmp + ((int64_t)row * a.stride_tmp_g + 16 * db + 4 * kg) * 2) = pk;
+    }
+  }
+}
+
+// Stage 2 for those head sizes: one wave per (sequence, kv head, output row); lane l owns head dims l, l + 64, ...
+template <int D>
+__global__ __launch_bounds__(64) void pa_reduce_generic_kernel(const PaDecodeArgs a) {
+  constexpr int DPL = D / 64;
+  const int lane = threadIdx.x;
+  const int Ge = a.q_len * a.group_size;
+  const uint32_t wid = blockIdx.x;
+  const int row = (int)(wid % (uint32_t)Ge);
+  const int h = (int)((wid / (uint32_t)Ge) % (uint32_t)a.num_kv_heads);
+  const int b = (int)(wid / (uint32_t)(Ge * a.num_kv_heads));
+  const int ctx = a.context_lens[b];
+  int n = (ctx + a.partition_size - 1) / a.partition_size;
+  n = n > a.max_num_partitions ? a.max_num_partitions : n;
+  const int qb = a.q_lens ? a.q_lens[b] : a.q_len;
+  const bool live = n > 0 && row < qb * a.group_size;
+  __bf16* out = (__bf16*)a.output + (int64_t)b * a.stride_out_s + (int64_t)(h * Ge + row) * a.stride_out_h;
+  if (!live) {
+    if (!(a.flags & PA_DECODE_FLAG_OUTPUT_ONLY) || n <= 0) {
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) out[lane + 64 * i] = (__bf16)0.f;
+    }
+    return;
+  }
+  const int64_t es = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + row;
+  const __bf16* tmp = (const __bf16*)a.tmp_output + (int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
+                      (int64_t)row * a.stride_tmp_g;
+  float M = a.sinks ? a.sinks[h * Ge + row] : -INFINITY;  // (the sink takes part in the maximum)
+  for (int p = 0; p < n; ++p) M = fmaxf(M, a.max_logits[es + (int64_t)p * a.stride_es_p]);
+  const float M_safe = M == -INFINITY ? 0.f : M;
+  float L = 0.f;
+  float o[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) o[i] = 0.f;
+  for (int p = 0; p < n; ++p) {
+    const float w = a.exp_sums[es + (int64_t)p * a.stride_es_p] *
+                    __expf(a.max_logits[es + (int64_t)p * a.stride_es_p] - M_safe);
+    L += w;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) o[i] += w * (float)tmp[(int64_t)p * a.stride_tmp_p + lane + 64 * i];
+  }
+  if (a.sinks) L += __expf(a.sinks[h * Ge + row] - M_safe);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) out[lane + 64 * i] = (__bf16)(o[i] * inv);
+}
+
+}  // namespace
+
+#endif  // PA_GENERIC_KERNEL_H_

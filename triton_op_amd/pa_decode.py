@@ -195,8 +195,8 @@ def plan_decode(
         raise ValueError(f"equivalent_query_group_size_pow2={ge_pow2} exceeds maximum of 64")
     if block_size not in _SUPPORTED_BLOCK_SIZES:
         raise ValueError(f"kv_block_size == {block_size} not in {list(_SUPPORTED_BLOCK_SIZES)}")
-    if head_size != 128:
-        raise ValueError(f"head_size == {head_size} is not supported (128 only)")
+    if head_size not in (64, 128, 256):  # (128 on the tuned kernels, 64 and 256 on the generic ones)
+        raise ValueError(f"head_size == {head_size} is not supported (64, 128 or 256)")
     x = 16 // key_cache.element_size()
     if key_cache.shape[-1] != x or key_cache.shape[2] * x != head_size:
         raise ValueError(f"key_cache shape {tuple(key_cache.shape)} is not [blocks, kv_heads, {head_size}//{x}, bs, {x}]")
@@ -294,6 +294,13 @@ def plan_decode(
         elif num_sequence_partitions and num_sequence_partitions > 0:
             per = -(-max_seq // int(num_sequence_partitions))
             partition_size = -(-per // PARTITION_GRANULE) * PARTITION_GRANULE
+        elif head_size != 128:
+            # the generic kernels run one wave per (sequence, partition, kv head, 16-row tile): the shortest partitions
+            # that still leave the launch under a few dozen waves per SIMD
+            partition_size = PARTITION_GRANULE
+            while (num_seqs * num_kv_heads * -(-ge // 16) * -(-max_seq // partition_size) > 32768
+                   and partition_size < 4096):
+                partition_size *= 2
         else:
             partition_size = select_partition_size(num_seqs, num_kv_heads, ge, max_seq, block_size, 0,
                                                    int(total_context_tokens))
