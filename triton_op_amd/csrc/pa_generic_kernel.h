@@ -15,7 +15,7 @@ namespace {
 // Stage 1: one wave per (sequence, partition, kv head, 16-row query tile).  A 64-token step is four 16-token
 // tiles.  v_mfma_f32_16x16x16_bf16 holds, in lane l (li = l % 16, kg = l / 16), four consecutive reduction indices
 // 4 kg .. 4 kg + 3 of row / column li of its operands and rows 4 kg .. 4 kg + 3 of column li of its result, so:
-//   S^T[token, row] = K Q^T:  A = 4 head dims of token li (4 or 8 bytes of the cache, converted to bf16),
+//   S^T[token, row] = K Q^T:  A = 4 head dims of token li (a quarter of a 16-byte piece of the cache, as bf16),
 //                             B = the same 4 head dims of query row li; the result holds 4 tokens of row li;
 //   O^T[dim, row]   = V^T P:  A = 4 tokens of head dim li of a 16-dim block, B = P of those 4 tokens for row li --
 //                             exactly what the lane holds of S^T, so P never moves between lanes.
@@ -96,15 +96,18 @@ void pa_partition_generic_kernel(const PaDecodeArgs a) {
   float slope2 = 0.f;
   if (a.alibi_slopes && row_ok)
     slope2 = a.alibi_slopes[a.alibi_slopes_len == Hkv * Ge ? h * Ge + row : h * G + (row - t_row * G)] * kLog2e;
+  // (the order of the reduction index is free as long as both operands agree: MFMA c = 4 g + m takes head dims
+  // 64 g + 16 kg + 4 m .. + 3 from lane group kg, so a lane's K bytes of four MFMAs are ONE 16-byte piece of the cache)
   bf16x4_bits qreg[DB];
   {
-    const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (row_ok ? row : 0)) * a.stride_q_h + 4 * kg;
+    const int64_t e0 = (int64_t)b * a.stride_q_s + (int64_t)(h * Ge + (row_ok ? row : 0)) * a.stride_q_h + 16 * kg;
 #pragma unroll
     for (int c = 0; c < DB; ++c) {
+      const int d = 64 * (c >> 2) + 4 * (c & 3);
       if (a.query_dtype == PA_DTYPE_BF16)
-        qreg[c] = load_cache4<false>((const char*)a.query + (e0 + 16 * c) * 2);
+        qreg[c] = load_cache4<false>((const char*)a.query + (e0 + d) * 2);
       else
-        qreg[c] = load_cache4<true>((const char*)a.query + (e0 + 16 * c));
+        qreg[c] = load_cache4<true>((const char*)a.query + (e0 + d));
       if (!row_ok) qreg[c] = bf16x4_bits{0, 0, 0, 0};
     }
   }
@@ -138,11 +141,33 @@ void pa_partition_generic_kernel(const PaDecodeArgs a) {
       s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
       const char* kt = kbase + (int64_t)page[j] * a.stride_k_b * ESZ;
 #pragma unroll
-      for (int c = 0; c < DB; ++c) {
-        const int d = 16 * c + 4 * kg;  // this lane's four head dims: inside one chunk of X dims
-        const bf16x4_bits ka =
-            load_cache4<FP8>(kt + ((int64_t)(d / X) * a.stride_k_c + (off[j] + li) * X + d % X) * ESZ);
-        s[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka, qreg[c], s[j], 0, 0, 0);
+      for (int g = 0; g < D / 64; ++g) {
+        // this lane's 16 head dims of the 64-dim group: one 16-byte piece (FP8) or two (bf16)
+        union {
+          u32x4 q[2];
+          uint32_t u[8];
+        } kv;
+        if constexpr (FP8) {
+          kv.q[0] = load16(kt + (int64_t)(4 * g + kg) * a.stride_k_c + (off[j] + li) * 16);
+        } else {
+          kv.q[0] = load16(kt + ((int64_t)(8 * g + 2 * kg) * a.stride_k_c + (off[j] + li) * 8) * 2);
+          kv.q[1] = load16(kt + ((int64_t)(8 * g + 2 * kg + 1) * a.stride_k_c + (off[j] + li) * 8) * 2);
+        }
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          union {
+            bf16x4_bits v;
+            uint32_t u[2];
+          } ka;
+          if constexpr (FP8) {
+            ka.u[0] = fp8x2_to_bf16x2(kv.u[m], false);
+            ka.u[1] = fp8x2_to_bf16x2(kv.u[m], true);
+          } else {
+            ka.u[0] = kv.u[2 * m];
+            ka.u[1] = kv.u[2 * m + 1];
+          }
+          s[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka.v, qreg[4 * g + m], s[j], 0, 0, 0);
+        }
       }
     }
     // ---- scales, ALiBi, mask; row maximum ---------------------------------------------------------------------------
