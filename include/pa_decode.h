@@ -270,7 +270,7 @@ typedef struct PaKvWriteArgs {
   float* value_scale;
   int64_t num_tokens;
   int32_t num_kv_heads;
-  int32_t head_size;           /* 128 */
+  int32_t head_size;           /* 128; 64 and 256 are written token by token whatever num_tokens is */
   int32_t block_size;
   int32_t cache_dtype;         /* PA_DTYPE_* */
   int32_t kv_quant_mode;       /* PA_QUANT_* */

@@ -28,34 +28,51 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 // element index of (head dim d, token offset off) inside one (block, head) of the V cache: rows of block_size
 // tokens per head dim, or, transposed, tiles of X tokens (X = 16 / element size) with the head dims inside a tile
-template <int X>
+template <int X, int D = 128>
 __device__ __forceinline__ int64_t v_index(const PaKvWriteArgs& a, int d, int off) {
-  return a.v_transposed ? ((int64_t)(off / X) * 128 + d) * X + off % X : (int64_t)d * a.block_size + off;
+  return a.v_transposed ? ((int64_t)(off / X) * D + d) * X + off % X : (int64_t)d * a.block_size + off;
 }
 
-// ---- one (token, kv head) by one wave; lane l owns head dims 2l, 2l+1 ----------------------------------------
-template <bool TO_FP8>
+// ---- one (token, kv head) by one wave; lane l owns head dims 2l, 2l+1 (+ 128 per further pass: head size 256 takes
+// two passes, head size 64 uses half the lanes) ---------------------------------------------------------------------
+template <bool TO_FP8, int D = 128>
 __device__ __forceinline__ void write_token(const PaKvWriteArgs& a, long long t, int h, long long slot, int lane) {
+  constexpr int PASSES = (D + 127) / 128;
   const long long block = slot / a.block_size;
   const int off = (int)(slot - block * a.block_size);
   const int bs = a.block_size;
 
-  const uint32_t kraw = *reinterpret_cast<const uint32_t*>((const uint16_t*)a.key + t * a.stride_k_t + h * a.stride_k_h + 2 * lane);
-  const uint32_t vraw = *reinterpret_cast<const uint32_t*>((const uint16_t*)a.value + t * a.stride_v_t + h * a.stride_v_h + 2 * lane);
-  const int d0 = 2 * lane;
+  uint32_t kraw[PASSES], vraw[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int d0 = 128 * p + 2 * lane;
+    kraw[p] = vraw[p] = 0u;
+    if (d0 < D) {
+      kraw[p] = *reinterpret_cast<const uint32_t*>((const uint16_t*)a.key + t * a.stride_k_t + h * a.stride_k_h + d0);
+      vraw[p] = *reinterpret_cast<const uint32_t*>((const uint16_t*)a.value + t * a.stride_v_t + h * a.stride_v_h + d0);
+    }
+  }
   if constexpr (!TO_FP8) {
     // 16-bit cache: x = 8; the two dims of a lane are adjacent in a chunk
     uint16_t* kc = (uint16_t*)a.key_cache + block * a.stride_kc_b + h * a.stride_kc_h;
-    *reinterpret_cast<uint32_t*>(kc + (int64_t)(d0 / 8) * bs * 8 + off * 8 + d0 % 8) = kraw;
     uint16_t* vc = (uint16_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
-    vc[v_index<8>(a, d0, off)] = (uint16_t)(vraw & 0xffffu);
-    vc[v_index<8>(a, d0 + 1, off)] = (uint16_t)(vraw >> 16);
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int d0 = 128 * p + 2 * lane;
+      if (d0 >= D) continue;
+      *reinterpret_cast<uint32_t*>(kc + (int64_t)(d0 / 8) * bs * 8 + off * 8 + d0 % 8) = kraw[p];
+      vc[v_index<8, D>(a, d0, off)] = (uint16_t)(vraw[p] & 0xffffu);
+      vc[v_index<8, D>(a, d0 + 1, off)] = (uint16_t)(vraw[p] >> 16);
+    }
   } else {
-    const float k0 = bf16_to_f32(kraw & 0xffffu), k1 = bf16_to_f32(kraw >> 16);
-    const float v0 = bf16_to_f32(vraw & 0xffffu), v1 = bf16_to_f32(vraw >> 16);
     float ks, vs;
     if (a.kv_quant_mode == PA_QUANT_PER_TOKEN) {
-      float ka = fmaxf(fabsf(k0), fabsf(k1)), va = fmaxf(fabsf(v0), fabsf(v1));
+      float ka = 0.f, va = 0.f;
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        ka = fmaxf(ka, fmaxf(fabsf(bf16_to_f32(kraw[p] & 0xffffu)), fabsf(bf16_to_f32(kraw[p] >> 16))));
+        va = fmaxf(va, fmaxf(fabsf(bf16_to_f32(vraw[p] & 0xffffu)), fabsf(bf16_to_f32(vraw[p] >> 16))));
+      }
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) {
         ka = fmaxf(ka, __shfl_xor(ka, o));
@@ -74,18 +91,25 @@ __device__ __forceinline__ void write_token(const PaKvWriteArgs& a, long long t,
     } else {
       ks = vs = 1.f;
     }
-    const uint8_t qk0 = f32_to_fp8(__fdiv_rn(k0, ks)), qk1 = f32_to_fp8(__fdiv_rn(k1, ks));
-    const uint8_t qv0 = f32_to_fp8(__fdiv_rn(v0, vs)), qv1 = f32_to_fp8(__fdiv_rn(v1, vs));
     uint8_t* kc = (uint8_t*)a.key_cache + block * a.stride_kc_b + h * a.stride_kc_h;
-    *reinterpret_cast<uint16_t*>(kc + (int64_t)(d0 / 16) * bs * 16 + off * 16 + d0 % 16) = (uint16_t)(qk0 | (qk1 << 8));
     uint8_t* vc = (uint8_t*)a.value_cache + block * a.stride_vc_b + h * a.stride_vc_h;
-    vc[v_index<16>(a, d0, off)] = qv0;
-    vc[v_index<16>(a, d0 + 1, off)] = qv1;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int d0 = 128 * p + 2 * lane;
+      if (d0 >= D) continue;
+      const float k0 = bf16_to_f32(kraw[p] & 0xffffu), k1 = bf16_to_f32(kraw[p] >> 16);
+      const float v0 = bf16_to_f32(vraw[p] & 0xffffu), v1 = bf16_to_f32(vraw[p] >> 16);
+      const uint8_t qk0 = f32_to_fp8(__fdiv_rn(k0, ks)), qk1 = f32_to_fp8(__fdiv_rn(k1, ks));
+      const uint8_t qv0 = f32_to_fp8(__fdiv_rn(v0, vs)), qv1 = f32_to_fp8(__fdiv_rn(v1, vs));
+      *reinterpret_cast<uint16_t*>(kc + (int64_t)(d0 / 16) * bs * 16 + off * 16 + d0 % 16) = (uint16_t)(qk0 | (qk1 << 8));
+      vc[v_index<16, D>(a, d0, off)] = qv0;
+      vc[v_index<16, D>(a, d0 + 1, off)] = qv1;
+    }
   }
 }
 
 // ---- append, a few tokens (decode): one wave per (token, kv head) ------------------------------------------------
-template <bool TO_FP8>
+template <bool TO_FP8, int D = 128>
 __global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs a) {
   const int lane = threadIdx.x & 63;
   const long long item = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -94,7 +118,7 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(const PaKvWriteArgs
   const long long t = item / a.num_kv_heads;
   const long long slot = a.slot_mapping[t];
   if (slot < 0) return;  // padding token
-  write_token<TO_FP8>(a, t, h, slot, lane);
+  write_token<TO_FP8, D>(a, t, h, slot, lane);
 }
 
 // lane exchanges inside a row of 16 lanes on the vector ALU (DPP), not through the LDS crossbar
@@ -485,7 +509,7 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
   if (a->struct_size != sizeof(PaKvWriteArgs)) return PA_ERR_BAD_STRUCT;
   if (!a->key || !a->value || !a->slot_mapping || !a->key_cache || !a->value_cache) return PA_ERR_NULL_POINTER;
   if (a->num_tokens < 0 || a->num_kv_heads <= 0 || a->block_size <= 0) return PA_ERR_BAD_SHAPE;
-  if (a->head_size != 128) return PA_ERR_UNSUPPORTED;
+  if (a->head_size != 128 && a->head_size != 64 && a->head_size != 256) return PA_ERR_UNSUPPORTED;
   if (a->cache_dtype != PA_DTYPE_BF16 && a->cache_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
   if (a->v_transposed != 0 && a->v_transposed != 1) return PA_ERR_BAD_SHAPE;
   if (a->v_transposed && a->block_size % (a->cache_dtype == PA_DTYPE_FP8_E4M3FN ? 16 : 8)) return PA_ERR_BAD_SHAPE;
@@ -505,6 +529,15 @@ int pa_kv_cache_write(const PaKvWriteArgs* a, void* hip_stream) {
                         ((reinterpret_cast<uintptr_t>(a->key_cache) | reinterpret_cast<uintptr_t>(a->value_cache)) & 15) == 0 &&
                         a->stride_kc_b % 16 == 0 && a->stride_kc_h % 16 == 0 && a->stride_vc_b % 16 == 0 && a->stride_vc_h % 16 == 0 &&
                         a->block_size % 16 == 0;
+  if (a->head_size != 128) {  // head sizes 64 and 256: token by token, whatever the number of tokens
+    const dim3 grid((unsigned)blocks), block(256);
+    const bool fp8 = a->cache_dtype == PA_DTYPE_FP8_E4M3FN;
+    if (a->head_size == 64)
+      return fp8 ? pa_launch(kv_cache_write_kernel<true, 64>, grid, block, 0, stream, *a)
+                 : pa_launch(kv_cache_write_kernel<false, 64>, grid, block, 0, stream, *a);
+    return fp8 ? pa_launch(kv_cache_write_kernel<true, 256>, grid, block, 0, stream, *a)
+               : pa_launch(kv_cache_write_kernel<false, 256>, grid, block, 0, stream, *a);
+  }
   if (rows_16b && a->num_tokens >= 2048) {
     const int regroup = a->block_size > 16;
     const int bs_shift = (a->block_size & (a->block_size - 1)) == 0 ? __builtin_ctz((unsigned)a->block_size) : -1;
