@@ -16,8 +16,8 @@ extern "C" {
 
 /*
  * A read-only probe of the memory access pattern of stage 1.  For the same arguments it reads the K and V bytes
- * that the partition kernel for up to 16 query rows reads (FP8 cache, block size 16, dense layout; anything else
- * is PA_ERR_UNSUPPORTED), with the same workgroup decomposition, load width and cache policy, and does no
+ * that the partition kernel for up to 16 query rows reads (FP8 cache, plain V layout, any power-of-two block size;
+ * anything else is PA_ERR_UNSUPPORTED), with the same workgroup decomposition, load width and cache policy, and does no
  * arithmetic: its duration is what the memory system gives the gather pattern.  sink: at least 64 int32 of device
  * memory (written only in a case that does not occur; it keeps the loads alive).
  */

@@ -26,13 +26,17 @@ int pa_probe_gather(const PaDecodeArgs* a, int32_t* sink, void* hip_stream) {
   if (a->num_seqs <= 0 || a->num_kv_heads <= 0 || a->max_num_partitions <= 0 || a->partition_size <= 0 ||
       a->partition_size % 256)
     return PA_ERR_BAD_SHAPE;
-  if (a->kv_dtype != PA_DTYPE_FP8_E4M3FN || a->block_size != 16 || a->stride_k_c != 256 || a->stride_v_2 != 16 ||
+  if (a->kv_dtype != PA_DTYPE_FP8_E4M3FN || a->block_size < 16 || (a->block_size & (a->block_size - 1)) ||
       a->v_transposed || a->head_size != kHeadSize)
     return PA_ERR_UNSUPPORTED;
   const long long blocks = (long long)a->num_seqs * a->num_kv_heads * a->max_num_partitions;
   if (blocks > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
-  return launch(pa_gather_probe_kernel, dim3((unsigned)blocks), dim3(256), reinterpret_cast<hipStream_t>(hip_stream), *a,
-                reinterpret_cast<int*>(sink));
+  const bool bs16 = a->block_size == 16 && a->stride_k_c == 256 && a->stride_v_2 == 16;
+  if (bs16)
+    return launch(pa_gather_probe_kernel<true>, dim3((unsigned)blocks), dim3(256), reinterpret_cast<hipStream_t>(hip_stream),
+                  *a, reinterpret_cast<int*>(sink));
+  return launch(pa_gather_probe_kernel<false>, dim3((unsigned)blocks), dim3(256), reinterpret_cast<hipStream_t>(hip_stream),
+                *a, reinterpret_cast<int*>(sink));
 }
 
 int pa_probe_stream(const PaDecodeArgs* a, int32_t depth, int32_t workgroups_per_cu, int32_t variant, int32_t* sink,

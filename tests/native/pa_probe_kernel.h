@@ -15,6 +15,7 @@ namespace {
 // and the partition kernel is what the kernel's arithmetic and its tail cost.
 // Block size 16, FP8 cache in the dense default layout only.  `sink` receives a word only if the fold of all the
 // bytes read is a value it cannot be (which keeps the loads alive without a store per workgroup).
+template <bool BS16>  // block size 16 in the dense layout: constant in-page strides, as in the kernel's own variant
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void pa_gather_probe_kernel(const PaDecodeArgs a, int* sink) {
   const int lane = threadIdx.x & 63;
@@ -37,29 +38,43 @@ void pa_gather_probe_kernel(const PaDecodeArgs a, int* sink) {
   const char* vbase = (const char*)a.value_cache + (int64_t)h * a.stride_v_h;
   const int* bt = a.block_tables + (int64_t)b * a.stride_bt_s;
   const int last_tile_tok = (wg_end - 1) & ~15;
-  const uint32_t k_off = (uint32_t)(kg * 256 + li * 16);
+  // (any block size and the plain V layout: the strides come from the arguments; with pages of more than 64 tokens
+  // the V rows are read with ordinary loads, as the kernel reads them: a step takes half a 128-byte line of a row)
+  const int log2_bs = BS16 ? 4 : 31 - __builtin_clz(a.block_size);
+  const int bs_mask = BS16 ? 15 : a.block_size - 1;
+  const uint32_t k_chunk = BS16 ? 256u : (uint32_t)a.stride_k_c;
+  const uint32_t k_off = (uint32_t)(kg * k_chunk + li * 16);
+  const uint32_t v_row = BS16 ? 16u : (uint32_t)a.stride_v_2;
+  const bool v_stream = BS16 || a.block_size <= 64;
   struct Step {
     u32x4 k[4][2];
     u32x4 v[8];
   };
   auto issue = [&](Step& st, int tok0) {
-    int page[4];
+    int page[4], off[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int t = tok0 + 16 * j;
       t = t > last_tile_tok ? last_tile_tok : t;
-      page[j] = sload_i32(bt + (t >> 4));
+      page[j] = sload_i32(bt + (t >> log2_bs));
+      off[j] = t & bs_mask;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const char* tb = kbase + (int64_t)page[j] * a.stride_k_b;
+      const char* tb = kbase + (int64_t)page[j] * a.stride_k_b + (int64_t)off[j] * 16;
       st.k[j][0] = load16_stream(tb + k_off);
-      st.k[j][1] = load16_stream(tb + k_off + 1024);
+      st.k[j][1] = load16_stream(tb + k_off + 4 * k_chunk);
     }
     const int vp = kg == 0 ? page[0] : (kg == 1 ? page[1] : (kg == 2 ? page[2] : page[3]));
-    const char* tb = vbase + (int64_t)vp * a.stride_v_b;
+    const int vo = kg == 0 ? off[0] : (kg == 1 ? off[1] : (kg == 2 ? off[2] : off[3]));
+    const char* tb = vbase + (int64_t)vp * a.stride_v_b + vo;
+    if (v_stream) {
 #pragma unroll
-    for (int db = 0; db < 8; ++db) st.v[db] = load16_stream(tb + (li + 16 * db) * 16);
+      for (int db = 0; db < 8; ++db) st.v[db] = load16_stream(tb + (li + 16 * db) * v_row);
+    } else {
+#pragma unroll
+      for (int db = 0; db < 8; ++db) st.v[db] = load16(tb + (li + 16 * db) * v_row);
+    }
   };
   uint32_t fold = 0;
   auto consume = [&](const Step& st) {
