@@ -808,7 +808,7 @@ def _adversarial(wl, kind):
     return wl, slopes
 
 
-@pytest.mark.parametrize("rows", ["g8_q1", "g8_q4", "g16_q4", "g16_q3_bs1024"])
+@pytest.mark.parametrize("rows", ["g8_q1", "g8_q4", "g16_q4", "g16_q3_bs1024", "g8_q4_head64", "g16_q4_head256"])
 @pytest.mark.parametrize("kind", ["gain64", "alibi2", "kscale_waves", "vscales", "gain64_vscales", "vscales_rising",
                                   "vscales_falling_logits_rising"])
 def test_adversarial_softmax_levels(cuda, kind, rows):
@@ -819,9 +819,11 @@ def test_adversarial_softmax_levels(cuda, kind, rows):
     kernel with two waves per row tile, 64 and 48 rows with one (reference maximum that is re-based).  Every output
     must be finite and meet the oracle at the usual bar, measured against each row's own magnitude (the outputs
     reach 2^40); the partition buffers are held against the oracle's partition stage."""
-    g, q_len, bs = dict(g8_q1=(8, 1, 16), g8_q4=(8, 4, 16), g16_q4=(16, 4, 16), g16_q3_bs1024=(16, 3, 1024))[rows]
+    g, q_len, bs, hd = dict(g8_q1=(8, 1, 16, 128), g8_q4=(8, 4, 16, 128), g16_q4=(16, 4, 16, 128),
+                            g16_q3_bs1024=(16, 3, 1024, 128), g8_q4_head64=(8, 4, 16, 64),
+                            g16_q4_head256=(16, 4, 16, 256))[rows]  # (the last two: the generic kernels)
     wl = _make(batch=3, num_q_heads=2 * g, num_kv_heads=2, context_lens=_ctx(2048, 700, 1030), q_len=q_len,
-               scale_mode="token", block_size=bs, seed=17)
+               scale_mode="token", block_size=bs, seed=17, head_size=hd)
     wl, slopes = _adversarial(wl, kind)
     ref = _oracle(wl, slopes).float()
     assert bool(torch.isfinite(ref).all())
