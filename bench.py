@@ -682,7 +682,12 @@ def _bench_trace(a) -> int:
     xcd_of = (np.arange(len(t)) & 7)[t[:, 5] > 0]  # workgroup ids go round the eight XCDs
     t = t[t[:, 5] > 0]
     us = 0.01  # per tick
-    ent, req, qry, first, last, end, steps, rows = [t[:, i] for i in range(8)]
+    ent, req, qry, first, last, end, steps = [t[:, i] for i in range(7)]
+    where = words.reshape(-1, 8)[:, 7][words.reshape(-1, 8)[:, 5] > 0]
+    rows = (where & np.uint64(0xffff)).astype(np.float64)
+    hw_id, xcc_id = ((where >> np.uint64(16)) & np.uint64(0xffff)).astype(np.int64), ((where >> np.uint64(32)) & np.uint64(0xf)).astype(np.int64)
+    # HW_ID: cu_id bits 8-11, sh_id bit 12, se_id bits 13-15: one number per CU of the GPU
+    cu_of = xcc_id * 4096 + ((hw_id >> 8) & 0xff)
     start, span = ent.min(), (end.max() - ent.min()) * us
     slots = int(plan.launch_info().split(" workgroups per CU")[0].split()[-1]) * torch.cuda.get_device_properties(dev).multi_processor_count
 
@@ -708,6 +713,14 @@ def _bench_trace(a) -> int:
         "xcd_end_us": [round(float((end[xcd_of == x].max() - start) * us), 1) for x in range(8)],
         "xcd_busy_per_slot_us": [round(float((end - ent)[xcd_of == x].sum() * us / (slots / 8)), 1) for x in range(8)],
         "xcd_per_step_us": [round(float((((last - first) / np.maximum(steps, 1))[(xcd_of == x) & (steps >= 16)]).mean() * us), 3) for x in range(8)],
+        # per CU: the mean time of a step over the CU's workgroups (16 steps or more): slowest, median and fastest CU
+        "cu_per_step_us": (lambda v: {"cus": len(v), "min": round(min(v), 3), "median": round(sorted(v)[len(v) // 2], 3),
+                                      "max": round(max(v), 3)})(
+            [float((((last - first) / np.maximum(steps, 1))[(cu_of == c) & (steps >= 16)]).mean() * us)
+             for c in np.unique(cu_of) if ((cu_of == c) & (steps >= 16)).any()]),
+        "cu_busy_us": (lambda v: {"min": round(min(v), 1), "median": round(sorted(v)[len(v) // 2], 1), "max": round(max(v), 1)})(
+            [float((end - ent)[cu_of == c].sum() * us / (slots / torch.cuda.get_device_properties(dev).multi_processor_count))
+             for c in np.unique(cu_of)]),
         "per_step_us_by_live_rows": {str(r): round(float((((last - first) / steps)[(rows > r - 16) & (rows <= r) & (steps >= 16)]).mean() * us), 2)
                                      for r in (16, 32, 48, 64) if ((rows > r - 16) & (rows <= r) & (steps >= 16)).any()},
     }, ensure_ascii=False))

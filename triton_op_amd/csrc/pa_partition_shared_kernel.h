@@ -666,7 +666,10 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
     for (int i = 0; i < 5; ++i) t[i] = pa_trace_t[i];
     t[5] = wall_clock64();
     t[6] = (unsigned long long)n_steps;
-    t[7] = (unsigned long long)rows_valid;
+    // live rows, and where the workgroup ran: HW_ID (CU, shader array, shader engine) and XCC_ID
+    const unsigned hw = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_REG_HW_ID, 32 bits
+    const unsigned xcc = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)); // HW_REG_XCC_ID
+    t[7] = (unsigned long long)rows_valid | ((unsigned long long)(hw & 0xffffu) << 16) | ((unsigned long long)(xcc & 0xfu) << 32);
   }
 #endif
 }
