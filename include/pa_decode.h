@@ -145,7 +145,7 @@ typedef struct PaDecodeArgs {
   int64_t stride_q_s, stride_q_h;
   int64_t stride_k_b, stride_k_h, stride_k_c;     /* block, kv head, 16-byte chunk row */
   int64_t stride_v_b, stride_v_h, stride_v_2;     /* block, kv head, dim 2 (D rows, or bs/x rows) */
-  int64_t stride_bt_s;
+  int64_t stride_bt_s;                            /* >= the number of entries of a row (rows do not overlap) */
   int64_t stride_es_s, stride_es_h, stride_es_p;  /* shared by exp_sums and max_logits */
   int64_t stride_tmp_s, stride_tmp_h, stride_tmp_p, stride_tmp_g;
   int64_t stride_qscale_s;                        /* per-token query scale: stride of dim 0 */

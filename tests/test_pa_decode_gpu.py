@@ -643,7 +643,7 @@ def test_c_abi_rejects_bad_arguments(cuda, pa_lib):
                          wl.softmax_scale, 1, 300, torch.bfloat16, None, wl.key_scale, wl.value_scale)
     a = plan.args
     assert pa_lib.pa_decode(None, None) == -1
-    for field, bad, code in (("struct_size", 8, -2), ("head_size", 96, -3), ("block_size", 32, -3),
+    for field, bad, code in (("struct_size", 8, -2), ("head_size", 96, -3), ("block_size", 32, -3), ("stride_bt_s", 0, -4),
                              ("partition_size", 100, -4), ("key_cache", None, -1), ("num_seqs", 0, -4),
                              ("stride_k_b", 8, -4)):
         good = getattr(a, field)
@@ -1134,3 +1134,25 @@ def test_head_sizes_64_and_256_options(cuda, head_size, feature):
             assert torch.all(view(got)[b, :, ql:] == 7.0)
     if feature != "output_only":
         torch.testing.assert_close(got, ref.float(), atol=ATOL, rtol=RTOL)
+
+
+@pytest.mark.parametrize("num_q_heads,q_len", [(16, 1), (32, 4)])
+def test_one_block_table_row_expanded_over_the_batch(cuda, num_q_heads, q_len):
+    """Sequences that share their pages through ONE block-table row expanded over the batch (row stride 0): the entry
+    point gives every row a stride of its own (the kernels request a row's first entries before they know the
+    sequence's length and keep the index inside the row's stride; the C ABI refuses a stride below 1)."""
+    import triton_op_amd as T
+
+    wl = _make(batch=3, num_q_heads=num_q_heads, num_kv_heads=2, context_lens=_ctx(700, 700, 700), q_len=q_len,
+               scale_mode="token")
+    row = wl.block_tables[:1]
+    shared = type(wl)(**{**wl.__dict__, "block_tables": row.expand(3, -1), "context_lens": _ctx(700, 33, 300)})
+    g = shared.to(cuda)
+    bt = g.block_tables[:1].expand(3, -1)
+    assert bt.stride(0) == 0
+    out = torch.full_like(g.query, float("nan"))
+    T.paged_attention_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, bt, g.softmax_scale, g.q_len,
+                             g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=256)
+    torch.cuda.synchronize()
+    ref = _oracle(type(wl)(**{**shared.__dict__, "block_tables": row.expand(3, -1).contiguous()}))
+    torch.testing.assert_close(out.float().cpu(), ref.float(), atol=ATOL, rtol=RTOL)

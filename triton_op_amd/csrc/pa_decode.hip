@@ -362,6 +362,9 @@ int check_partition(const PaDecodeArgs* a) {
   int rc = check_common(a);
   if (rc) return rc;
   if (!a->query || !a->key_cache || !a->value_cache || !a->block_tables) return PA_ERR_NULL_POINTER;
+  // a sequence's block-table row is at least one entry long and rows do not overlap (the kernels request a row's
+  // first entries before they know how many of them the sequence uses, and keep the index inside the row's stride)
+  if (a->stride_bt_s < 1 || a->stride_bt_s > 0x7fffffffLL) return PA_ERR_BAD_SHAPE;
   if (a->block_size != 16 && a->block_size != 64 && a->block_size != 1024) return PA_ERR_UNSUPPORTED;
   if (a->kv_dtype != PA_DTYPE_BF16 && a->kv_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;
   if (a->query_dtype != PA_DTYPE_BF16 && a->query_dtype != PA_DTYPE_FP8_E4M3FN) return PA_ERR_UNSUPPORTED;

@@ -220,7 +220,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     int idx = (part * a.partition_size + wave * kStepTokens + 16 * j) >> log2_bs;
-    idx = idx < (int)a.stride_bt_s ? idx : (int)a.stride_bt_s - 1;
+    idx = idx < (int)a.stride_bt_s ? idx : (int)a.stride_bt_s - 1;  // (stride_bt_s >= 1: checked by the launch layer)
     early_page[j] = sload_i32(bt + idx);
   }
   const int ctx = sload_i32(a.context_lens + b);

@@ -96,7 +96,7 @@ void pa_partition_shared_kernel(const PaDecodeArgs a) {
 #pragma unroll
   for (int i = 0; i < NB - 1; ++i) {
     int idx = (part * a.partition_size + i * kStepTokens + 16 * wave) >> log2_bs;
-    idx = idx < (int)a.stride_bt_s ? idx : (int)a.stride_bt_s - 1;
+    idx = idx < (int)a.stride_bt_s ? idx : (int)a.stride_bt_s - 1;  // (stride_bt_s >= 1: checked by the launch layer)
     early_page[i] = sload_i32(bt + idx);
   }
   const int ctx = sload_i32(a.context_lens + b);

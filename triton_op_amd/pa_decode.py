@@ -219,6 +219,9 @@ def plan_decode(
         raise ValueError("the innermost cache dimensions must be dense")
     if query.stride(2) != 1 or output.stride(2) != 1 or block_tables.stride(1) != 1 or not sequence_lengths.is_contiguous():
         raise ValueError("query/output/block_tables must be contiguous in their last dimension")
+    if block_tables.stride(0) < max(1, block_tables.shape[1]):
+        # rows that overlap (one row expanded over the batch): the kernels want every row in a stride of its own
+        block_tables = block_tables.contiguous()
 
     # ---- quantisation modes (:1753-1790) ---------------------------------------------------------------
     q_mode, stride_qs = _cabi.PA_QUANT_NONE, 0
