@@ -6,7 +6,7 @@
     python bench.py --workload c1|c2|c3|c4|c5 [--partition-size N]   one configuration
     python bench.py --workload ref:B,Hq,Hkv,bs,qlen[,transv][,ctx=N]  one row of the reference harness's sweep
     python bench.py --workload custom:b=..,hq=..,hkv=..,q=..,ctx=..[,bs=..,scale=token|tensor,kv=fp8|bf16,qdtype=bf16|fp8,transv=0|1,hd=64|128|256]
-                               [,lens=c5[,qlens=c5|N][,pick=one|rest]]   c5's draw of context lengths (and of new tokens per sequence)
+                               [,lens=c5[,cap=N][,qlens=c5|N][,pick=one|rest]]   c5's draw of context lengths (and of new tokens per sequence)
     python bench.py --workload probe_gather                          read-only probe of c2's page-gather pattern
     python bench.py --workload probe_gather:c5                       ... of another workload's (plain order, four-wave workgroups)
     python bench.py --workload probe_stream42:c5                     the pages read by workgroups whose waves share each step
@@ -52,7 +52,8 @@ HBM_TRAFFIC = {
         "bytes": 541_400_000, "launch": "pa_partition_kernel<fp8, bs16, 4 waves> x 512",
         "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
     ("c2_fp8_b64_ctx4k", 256): {
-        "bytes": 556_600_000, "launch": "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 4 partitions per workgroup",
+        "bytes": 557_700_000,
+        "launch": "pa_partition_kernel<fp8, bs16, 1 waves> x 512, teams of 4 waves, 4 partitions per wave, no reduce kernel",
         "profile": "profiles/pa_partition_kernel_c2_hbm_traffic.md"},
     ("c3_fp8_mtp2_bs1024", 8192): {
         "bytes": 4_437_300_000, "launch": "pa_partition_kernel<fp8, strided, 4 waves> x 4096, sorted items",
@@ -140,7 +141,7 @@ def _make_custom_workload(spec, device, seed):
     scale, kvd, qd = kv.get("scale", "tensor"), kv.get("kv", "fp8"), kv.get("qdtype", "bf16")
     transv = kv.get("transv", "0") == "1"
     hd = int(kv.get("hd", 128))  # head size: 128 on the tuned kernels, 64 / 256 on the generic ones
-    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv", "lens", "qlens", "pick", "hd"}
+    unknown = set(kv) - {"b", "hq", "hkv", "q", "ctx", "bs", "scale", "kv", "qdtype", "transv", "lens", "qlens", "pick", "hd", "cap"}
     if unknown:
         raise ValueError(f"custom: unknown keys {sorted(unknown)}")
     ctx_lens, q_lens, tag = torch.full((b,), ctx, dtype=torch.int32), None, f"ctx{ctx}"
@@ -151,6 +152,9 @@ def _make_custom_workload(spec, device, seed):
         ctx_lens = W._lognormal_ctx(b, 2048, 1.0, 16, 65536, gen)
         drawn = torch.randint(1, 5, (b,), generator=gen, dtype=torch.int32)
         tag = "c5lens"
+        if "cap" in kv:  # cap=N: no context longer than N tokens
+            ctx_lens = torch.clamp(ctx_lens, max=int(kv["cap"]))
+            tag += f"_cap{kv['cap']}"
         if "qlens" in kv:
             q_lens = drawn if kv["qlens"] == "c5" else torch.full((b,), int(kv["qlens"]), dtype=torch.int32)
             q_lens = torch.clamp(q_lens, max=q)
@@ -276,14 +280,16 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
     # ---- the dominant kernel alone.  When the partition kernel is the whole call (one partition per sequence), one
     # event pair brackets `steps` back-to-back launches, which is what a kernel trace's average sees; otherwise other
     # kernels run in between and every launch gets an event pair of its own (which also brackets its dispatch).
-    solo = plans[0].args.max_num_partitions == 1
+    # (a launch in teams merges in the partition kernel: pa_decode is that one kernel, pa_decode_partition another launch)
+    team = "no reduce kernel" in cfg.launch
+    solo = plans[0].args.max_num_partitions == 1 or team
     r_us_avg = None
     if solo:
         k_launches = max(steps, 100)  # (a short run's 20 launches would mostly measure the first one's ramp)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         for i in range(k_launches):
-            rc = lib.pa_decode_partition(C.byref(plans[i % n].args), sh)
+            rc = (lib.pa_decode if team else lib.pa_decode_partition)(C.byref(plans[i % n].args), sh)
             if rc:
                 _cabi.check(rc, "pa_decode_partition")
         e1.record(stream)

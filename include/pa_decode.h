@@ -203,7 +203,10 @@ int pa_decode_partition(const PaDecodeArgs* args, void* hip_stream);
 int pa_decode_reduce(const PaDecodeArgs* args, void* hip_stream);
 
 /* Both stages back to back on one stream: the body of the reference's paged_attention_decode.  Stage 2
- * skips the sequences stage 1 has finished, and is not launched when max_num_partitions == 1 (no sinks). */
+ * skips the sequences stage 1 has finished, and is not launched when max_num_partitions == 1 (no sinks), nor when
+ * stage 1 runs in teams: for a small partition size on a batch that fits the GPU at once, one workgroup of four
+ * waves covers a (sequence, kv head)'s whole partition axis, writes its partition-buffer entries as stage 1 does and
+ * merges them into output itself (pa_decode_launch_info says "teams of 4 waves ... no reduce kernel"). */
 int pa_decode(const PaDecodeArgs* args, void* hip_stream);
 
 /*
@@ -211,7 +214,8 @@ int pa_decode(const PaDecodeArgs* args, void* hip_stream);
  * and where its workgroups take their items from, e.g.
  *   "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
  *   "pa_partition_shared_kernel<fp8 per-token, bs16, 3 ring slots, 3 workgroups per CU> x 6512, sorted items".
- * The choice is a function of the arguments and the device's CU count alone.  (The reference's counterpart is
+ * With a non-NULL output the text is pa_decode's launch; with output == NULL it is pa_decode_partition's (which forms
+ * no teams).  The choice is a function of the arguments and the device's CU count alone.  (The reference's counterpart is
  * the kernel selection in pa_decode_triton_gluon_fp8.py:1492-1509.)  Launches nothing.
  *
  * Limits of the two launch modes that need a workspace (beyond them the call is launched in plain order, with
@@ -220,8 +224,8 @@ int pa_decode(const PaDecodeArgs* args, void* hip_stream);
  *
  * Environment: none of the library's behaviour depends on environment variables unless the process was started
  * with PA_DECODE_DEBUG=1, which enables the tuning switches PA_DECODE_WAVES, PA_DECODE_ROW_TILES, PA_DECODE_SPAN,
- * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED, PA_DECODE_LDS_PAD, PA_DECODE_P_RESIDUAL and PA_DECODE_XCD (read
- * once, at the first launch).
+ * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED, PA_DECODE_LDS_PAD, PA_DECODE_P_RESIDUAL, PA_DECODE_XCD and
+ * PA_DECODE_TEAM (read once, at the first launch).
  */
 int pa_decode_launch_info(const PaDecodeArgs* args, char* text, int32_t text_bytes);
 

@@ -411,9 +411,25 @@ def test_launch_layer_choices(pa_lib):
 
     # c2: one partition, four waves, 64 x 8 workgroups, no item list
     assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=4096) == "pa_partition_kernel<fp8, bs16, 4 waves> x 512"
-    # c2 at the reference's partition size: 16 x 512 partitions for 2048 wave slots: one-wave workgroups of four each
+    # c2 at the reference's partition size: 16 x 512 partitions for 2048 wave slots: one-wave walkers of four each, and
+    # the four of a (sequence, kv head) in one workgroup that merges them itself
     assert info(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=256) == \
-        "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 4 partitions per workgroup"
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 512, teams of 4 waves, 4 partitions per wave, no reduce kernel"
+    # ... without an output (stage 1 alone forms no teams), with too few sequences to fill three quarters of the wave
+    # slots, or with more than fit the GPU at once: one-wave workgroups
+    a = _fake_args(b=64, hq=64, hkv=8, q=1, ctx=4096, ps=256)
+    a.output = None
+    buf = C.create_string_buffer(256)
+    assert pa_lib.pa_decode_launch_info(C.byref(a), buf, 256) == 0
+    assert buf.value.decode() == "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 4 partitions per workgroup"
+    assert info(b=40, hq=64, hkv=8, q=1, ctx=4096, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 2560, 2 partitions per workgroup"
+    assert info(b=72, hq=64, hkv=8, q=1, ctx=4096, ps=256) == \
+        "pa_partition_kernel<fp8, bs16, 1 waves> x 2304, 4 partitions per workgroup"
+    # 13 partitions: 4 + 4 + 4 + 1; per-token scales: the teams of a sequence on one XCD
+    assert info(b=56, hq=64, hkv=8, q=1, ctx=3200, ps=256, per_token=True) == \
+        "pa_partition_kernel<fp8 per-token, bs16, 1 waves> x 448, teams of 4 waves, 4 partitions per wave, no reduce kernel, " \
+        "an item's heads on one XCD"
     # ... of 1024 tokens: two each; and never more than the partition axis holds (3 partitions: one workgroup per sequence and head, four rounds of them: sorted)
     assert info(b=128, hq=64, hkv=8, q=1, ctx=4096, ps=1024) == \
         "pa_partition_kernel<fp8, bs16, 1 waves> x 2048, 2 partitions per workgroup"

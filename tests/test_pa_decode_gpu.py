@@ -478,6 +478,157 @@ def test_workgroups_that_walk_several_partitions(cuda, kv, scale_mode, group, q_
     torch.testing.assert_close(out.float().cpu()[live], _oracle(wl, slopes, seq_ids=live).float()[live], atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("scale_mode,group,q_len,ragged,block_size,ps,max_ctx,batch,per_wave,alibi",
+                         [("tensor", 8, 1, False, 16, 256, 4096, 64, 4, False),   # the reference's shape: 16 partitions, 4 per wave
+                          ("token", 8, 1, False, 16, 256, 4096, 64, 4, False),
+                          ("tensor", 16, 1, False, 16, 256, 4096, 48, 4, False),  # 16 rows: full-size slots; 384 teams
+                          ("token", 4, 4, True, 16, 256, 3200, 64, 4, False),     # 13 partitions: 4 + 4 + 4 + 1; padding rows
+                          ("tensor", 4, 2, False, 64, 256, 1100, 64, 2, True),    # 5 partitions: 2 + 2 + 1 and an idle wave
+                          ("token", 8, 2, False, 16, 512, 2048, 64, 1, False),    # 4 partitions: one each
+                          ("tensor", 2, 3, True, 1024, 512, 2048, 64, 1, True),
+                          ("tensor", 8, 1, False, 16, 256, 7000, 64, 7, False)])  # 28 partitions of 8 rows: 7 per wave
+@pytest.mark.parametrize("output_only", [False, True])
+def test_teams_merge_in_the_partition_kernel(cuda, scale_mode, group, q_len, ragged, block_size, ps, max_ctx, batch, per_wave,
+                                             alibi, output_only):
+    """A caller-fixed small partition size on a batch whose (sequence, kv head) units are all resident at once, four waves each: four
+    one-wave walkers share a workgroup, cover the sequence's whole partition axis between them and merge their partial
+    results into `output` themselves; pa_decode launches no reduce kernel (the launch layer says so).  Contexts end
+    on, before and after partition and walk boundaries, reach one partition only (written by the wave that finished
+    them), leave whole waves of a team without a partition, or are empty (zero rows).  The partition buffers are
+    held against the oracle's partition stage (with the output-only flag they are scratch and stay untouched), the
+    result against the oracle; a second call with the same arguments is bit-identical.  With attention sinks no teams
+    are formed."""
+    import triton_op_amd as T
+
+    gen = torch.Generator().manual_seed(61)
+    ctx = torch.randint(1, max_ctx + 1, (batch,), generator=gen, dtype=torch.int32)
+    edge = [1, ps - 1, ps, ps + 1, per_wave * ps, per_wave * ps + 1, 2 * per_wave * ps + 63, 3 * per_wave * ps, max_ctx, max_ctx - 1]
+    ctx[:len(edge)] = torch.tensor([min(max(e, 1), max_ctx) for e in edge], dtype=torch.int32)
+    ctx = torch.clamp(ctx, min=q_len)
+    q_lens = None
+    if ragged:
+        q_lens = torch.randint(1, q_len + 1, (batch,), generator=gen, dtype=torch.int32)
+        q_lens[:4] = torch.tensor([1, q_len, 2, 1], dtype=torch.int32)
+    wl = _make(batch=batch, num_q_heads=group * 8, num_kv_heads=8, context_lens=ctx, q_len=q_len, q_lens=q_lens,
+               kv_dtype="fp8", scale_mode=scale_mode, block_size=block_size)
+    ctx = ctx.clone()
+    ctx[13] = 0  # (the generator wants a page per sequence: declared empty afterwards)
+    wl = type(wl)(**{**wl.__dict__, "context_lens": ctx})
+    live = [b for b in range(batch) if int(ctx[b]) > 0]
+    g = wl.to(cuda)
+    out = torch.full_like(g.query, float("nan"))
+    slopes = torch.linspace(0.01, 0.3, wl.query.shape[1], dtype=torch.float32) if alibi else None
+    kw = dict(partition_size=ps, query_lens=g.q_lens, alibi_slopes=None if slopes is None else slopes.to(cuda))
+    plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                         q_len, max_ctx, torch.bfloat16, None, g.key_scale, g.value_scale, output_only=output_only, **kw)
+    P = -(-max_ctx // ps)
+    assert plan.args.max_num_partitions == P
+    info = plan.launch_info()
+    assert f"teams of 4 waves, {per_wave} partitions per wave, no reduce kernel" in info and f"x {batch * 8}," in info, info
+    plan.exp_sums.fill_(float("nan"))
+    plan.max_logits.fill_(float("nan"))
+    plan.tmp_output.fill_(float("nan"))
+    plan.run()
+    torch.cuda.synchronize()
+    first = out.clone()
+    rows = (torch.ones(batch, dtype=torch.int32) * q_len if q_lens is None else q_lens)
+    gml, ges, gto = plan.max_logits.cpu(), plan.exp_sums.cpu(), plan.tmp_output.float().cpu()
+    if output_only:
+        assert torch.isnan(gml).all() and torch.isnan(ges).all() and torch.isnan(gto).all()
+    else:
+        reach = (torch.arange(P)[None, :] * ps < ctx[:, None])  # [batch, P]
+        ml, es, to = O.partition_stage(
+            wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
+            wl.q_len if wl.q_lens is None else wl.q_lens, wl.key_scale, wl.value_scale, slopes, ps, P, q_max=wl.q_len)
+        sel = reach[:, None, :, None].expand_as(ml)
+        fin = torch.isfinite(ml) & sel
+        assert torch.equal(gml[sel & ~torch.isfinite(ml)], ml[sel & ~torch.isfinite(ml)])
+        torch.testing.assert_close(gml[fin], ml[fin], atol=5e-4, rtol=5e-5)
+        torch.testing.assert_close(ges[sel], es[sel], atol=5e-4, rtol=1e-3)
+        sel_o = reach[:, None, :, None, None].expand_as(to)
+        torch.testing.assert_close(gto[sel_o], to[sel_o], atol=ATOL, rtol=RTOL)
+    # rows of a sequence: [kv head, query position, head of the group]
+    by_pos = lambda t: t.float().cpu().view(batch, 8, q_len, group, -1)
+    want = by_pos(_oracle(wl, slopes, seq_ids=live))
+    got = by_pos(out)
+    for b in live:
+        n = int(rows[b])
+        assert not torch.isnan(got[b, :, :n]).any(), b
+        torch.testing.assert_close(got[b, :, :n], want[b, :, :n], atol=ATOL, rtol=RTOL)
+        if not output_only:
+            assert bool((got[b, :, n:] == 0).all()), b
+    assert bool((got[13] == 0).all())
+    out.fill_(float("nan"))
+    plan.run()
+    torch.cuda.synchronize()
+    keep = ~torch.isnan(first.float())
+    assert torch.equal(torch.isnan(out.float()), ~keep)
+    assert torch.equal(out.view(torch.int16)[keep], first.view(torch.int16)[keep])
+    # with attention sinks (here of no weight) no teams are formed; the reduce kernel agrees with the team's merge (the
+    # same bf16 partials, merged in another order of additions)
+    out2 = torch.full_like(g.query, float("nan"))
+    plan2 = T.plan_decode(out2, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                          q_len, max_ctx, torch.bfloat16, None, g.key_scale, g.value_scale,
+                          sinks=torch.full((g.query.shape[1],), -1e30, dtype=torch.float32, device=cuda), **kw)
+    assert "teams" not in plan2.launch_info(), plan2.launch_info()
+    plan2.run()
+    torch.cuda.synchronize()
+    got2 = by_pos(out2)
+    for b in live:
+        n = int(rows[b])
+        torch.testing.assert_close(got2[b, :, :n], got[b, :, :n], atol=2e-3, rtol=2e-2)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_teams_seeded_sweep(cuda, seed):
+    """Random shapes the launch layer gives to teams (384 to 512 (sequence, kv head) units, up to 16 rows, 4 to 32
+    partitions of 256 or 512 tokens, per-tensor or per-token scales, ragged query lengths, ALiBi, pages of 16 or 64
+    tokens), random context lengths from one token to the whole partition axis: the result against the oracle."""
+    import random
+
+    import triton_op_amd as T
+
+    rng = random.Random(9100 + seed)
+    hkv = rng.choice([4, 8])
+    batch = rng.randint(384 // hkv, 512 // hkv)
+    group, q_len = rng.choice([(8, 1), (4, 2), (2, 4), (16, 1), (4, 4), (8, 2), (1, 3), (5, 3), (3, 1)])
+    ge = group * q_len
+    ps = rng.choice([256, 256, 512])
+    per_wave_max = min(8 if ge <= 8 else 4, 2048 // ps)
+    p_min = -(-2048 // (batch * hkv))  # one wave per workgroup: as many items as wave slots
+    P = rng.randint(max(p_min, 2), 4 * per_wave_max)
+    max_ctx = P * ps - rng.randint(0, ps - 1)
+    block_size = rng.choice([16, 16, 64])
+    scale_mode = rng.choice(["tensor", "token"])
+    ragged = q_len > 1 and rng.random() < 0.5
+    alibi = rng.random() < 0.3
+    gen = torch.Generator().manual_seed(9100 + seed)
+    ctx = torch.randint(1, max_ctx + 1, (batch,), generator=gen, dtype=torch.int32)
+    ctx[0], ctx[1] = max_ctx, 1
+    ctx = torch.clamp(ctx, min=q_len)
+    q_lens = torch.randint(1, q_len + 1, (batch,), generator=gen, dtype=torch.int32) if ragged else None
+    wl = _make(batch=batch, num_q_heads=group * hkv, num_kv_heads=hkv, context_lens=ctx, q_len=q_len, q_lens=q_lens,
+               kv_dtype="fp8", scale_mode=scale_mode, block_size=block_size, seed=9100 + seed)
+    g = wl.to(cuda)
+    out = torch.full_like(g.query, float("nan"))
+    slopes = torch.linspace(0.01, 0.3, wl.query.shape[1], dtype=torch.float32) if alibi else None
+    plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                         q_len, max_ctx, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
+                         query_lens=g.q_lens, alibi_slopes=None if slopes is None else slopes.to(cuda))
+    case = f"seed {seed}: batch {batch} hkv {hkv} group {group} q_len {q_len} ps {ps} P {P} bs {block_size} {scale_mode}"
+    assert "teams of 4 waves" in plan.launch_info(), case + " -> " + plan.launch_info()
+    print(case, flush=True)
+    plan.run()
+    torch.cuda.synchronize()
+    by_pos = lambda t: t.float().cpu().view(batch, hkv, q_len, group, -1)
+    got, want = by_pos(out), by_pos(_oracle(wl, slopes))
+    for b in range(batch):
+        n = q_len if q_lens is None else int(q_lens[b])
+        assert not torch.isnan(got[b, :, :n]).any(), case
+        torch.testing.assert_close(got[b, :, :n], want[b, :, :n], atol=ATOL, rtol=RTOL, msg=lambda m: case + ": " + m)
+        assert bool((got[b, :, n:] == 0).all()), case
+
+
 @pytest.mark.parametrize("group,q_len,scale_mode", [(8, 1, "tensor"), (16, 3, "token")])
 def test_item_list_reused_by_the_next_layer(cuda, group, q_len, scale_mode):
     """Two layers of one decode step share the sequence lengths and a workspace: the second is told to reuse the

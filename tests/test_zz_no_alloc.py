@@ -33,7 +33,11 @@ def _workloads(dev):
     ctx_b = torch.tensor([1500, 17, 700], dtype=torch.int32)
     b = W.make_decode_workload(name="noalloc_b", seed=22, batch=3, num_q_heads=16, num_kv_heads=2, block_size=16,
                                context_lens=ctx_b, q_len=1).to(dev)
-    return [(a, 256), (b, 256)]
+    # ... and one whose (sequence, kv head) units run as teams that merge in the partition kernel (no reduce kernel)
+    ctx_c = torch.randint(1, 2049, (52,), generator=g, dtype=torch.int32)
+    c = W.make_decode_workload(name="noalloc_c", seed=24, batch=52, num_q_heads=64, num_kv_heads=8, block_size=16,
+                               context_lens=ctx_c, q_len=1).to(dev)
+    return [(a, 256), (b, 256), (c, 256)]
 
 
 def test_noalloc_matches_pa_decode_on_two_calls_in_a_row():
@@ -42,6 +46,9 @@ def test_noalloc_matches_pa_decode_on_two_calls_in_a_row():
     stream = torch.cuda.current_stream(dev)
     for wl, ps in _workloads(dev):
         print(f"[noalloc] {wl.name} batch={wl.batch} partition_size={ps}", flush=True)
+        if wl.name == "noalloc_c":
+            info = _plan(wl, torch.empty_like(wl.query), ps).launch_info()
+            assert "teams of 4 waves" in info, info
         ref = torch.full_like(wl.query, float("nan"))
         _plan(wl, ref, ps).run()
         out = torch.full_like(wl.query, float("nan"))
@@ -77,7 +84,7 @@ def test_noalloc_call_captured_in_a_graph_replays_to_the_same_bits():
     on a device asks the runtime for the scratch array's address); then a call is captured and replayed three
     times with eager work and host synchronisations in between, each replay held against pa_decode's result."""
     dev = torch.device("cuda:0")
-    (wl, ps), _ = _workloads(dev)
+    wl, ps = _workloads(dev)[0]
     ref = torch.full_like(wl.query, float("nan"))
     _plan(wl, ref, ps).run()
     out = torch.full_like(wl.query, float("nan"))

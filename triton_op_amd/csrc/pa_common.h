@@ -47,6 +47,7 @@ constexpr int kFlagHeadsShareXcd = 0x80000;
 // tile; a tile of up to 8 real rows stages only those (half the bytes) and may walk twice as many partitions
 constexpr int kSpanMax = 4;
 constexpr int kSpanMaxFewRows = 8;
+constexpr int kTeamWaves = 4;  // one-wave span walkers that share a workgroup and merge their partial results in it
 // Workspace layout (int32 words): [0], [1] counters of the queued launch, [2] number of listed items,
 // [16 + 2i], [17 + 2i] sequence and partition index of item i.
 constexpr int kPlanHeaderWords = 16;

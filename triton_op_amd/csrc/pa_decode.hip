@@ -129,6 +129,7 @@ struct LaunchChoice {
   int row_tiles;    // pa_partition_kernel: 16-row query tiles one workgroup computes in its pass over the pages (1 or 2)
   int per_cu;       // workgroups of this instantiation that fit a CU
   int span;         // consecutive partitions a one-wave workgroup walks in one pass (1: one partition per workgroup)
+  bool team;        // four one-wave span walkers per workgroup cover a sequence's whole partition axis and merge it themselves
   bool queue;       // a resident grid pulls live items from a counter in the workspace
   bool sorted;      // items come from the planning kernel's list in the workspace
   bool listed_reduce;  // ... and pa_decode's reduce stage walks the planning kernel's list of multi-partition sequences
@@ -136,7 +137,9 @@ struct LaunchChoice {
   long long blocks; // workgroups launched
 };
 
-LaunchChoice choose_launch(const PaDecodeArgs& a) {
+// `fused`: the call is pa_decode's (both stages, `output` is written): the partition kernel may finish sequences of
+// several partitions itself
+LaunchChoice choose_launch(const PaDecodeArgs& a, bool fused) {
   LaunchChoice c{};
   const int ge = a.q_len * a.group_size;
   c.fp8 = a.kv_dtype == PA_DTYPE_FP8_E4M3FN;
@@ -219,7 +222,29 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
     // (a tile of up to 8 real rows stages half the bytes per partition and may walk twice as many)
     const long long span_max = c.row_tiles == 1 && ge <= 8 ? kSpanMaxFewRows : kSpanMax;
     span = span > span_max ? span_max : span;
-    if (span >= 2) {
+    // A TEAM: when four such walkers cover the whole partition axis they share a workgroup, which then holds every
+    // partial result of its (sequence, kv head, row tile) in LDS and merges them into `output` itself: no second
+    // kernel.  Only when every team is resident at once (two per CU) and the teams' waves fill three quarters of the
+    // wave slots or more: in a second round a team's waves would each have half the work of the one-wave workgroups
+    // that fill the slots in one (measured, 128 sequences x 8 kv heads x 1024 tokens at 256: 53.1 against 52.3 us;
+    // ragged, up to 8192 tokens: 198 against 183 us), and fewer teams lose to more, shorter workgroups (40 sequences x
+    // 8 x 4096 at 256: 70.3 against 67.8 us).  Measured, call against call with the reduce kernel: 64 x 8 x 4096 at
+    // 256: 93.2 -> 89.1 us; per-token scales, 56 sequences: 96.2 -> 84.3; 16 rows: 100.6 -> 95.9; 48 sequences: 75.6 ->
+    // 73.5; ragged, up to 4096 tokens: 67.3 -> 65.0; 64 x 8 x 1024: 29.4 -> 28.0; 64 x 8 x 7000: 157.7 -> 157.1.
+    // PA_DECODE_TEAM=0: never.
+    static const bool team_off = debug_switch("PA_DECODE_TEAM", 1) == 0;
+    const long long team_span = (a.max_num_partitions + kTeamWaves - 1) / kTeamWaves;
+    const long long teams = items / a.max_num_partitions;
+    if (fused && !team_off && c.fp8 && c.row_tiles == 1 && !a.sinks && a.output != nullptr && team_span <= span_max &&
+        team_span * a.partition_size <= 2048 && !(a.block_size > 64 && a.partition_size < 512 && team_span > 1) &&
+        forced_span != 1 && teams * kTeamWaves <= slots && teams * kTeamWaves * 4 >= slots * 3)
+    {
+      c.team = true;
+      c.span = (int)team_span;
+      c.per_cu = 2;
+      items = teams;
+      c.blocks = items;
+    } else if (span >= 2) {
       c.span = (int)span;
       const long long coarse = (a.max_num_partitions + span - 1) / span;
       items = items / a.max_num_partitions * coarse;
@@ -231,7 +256,7 @@ LaunchChoice choose_launch(const PaDecodeArgs& a) {
   // and the caller's workspace has room for the list (batches of more than kPlanMaxSeqs sequences, the planning
   // kernel's LDS tables, are launched in plain order).
   static const int sorted_mode = debug_switch("PA_DECODE_SORTED", -1);
-  c.sorted = !c.queue && sorted_mode != 0 && a.workspace != nullptr && a.num_seqs <= kPlanMaxSeqs &&
+  c.sorted = !c.queue && !c.team && sorted_mode != 0 && a.workspace != nullptr && a.num_seqs <= kPlanMaxSeqs &&
              a.workspace_bytes >= plan_workspace_bytes(a.num_seqs, a.max_num_partitions) &&
              (sorted_mode == 1 || items > 2LL * device_num_cus() * c.per_cu);
   // (with several partitions per workgroup the planning kernel lists those coarser items, and its list of the
@@ -263,6 +288,10 @@ int launch_partition_w(const PaDecodeArgs& k, const LaunchChoice& c, hipStream_t
     if (k.q_len * k.group_size > 32)
       return c.queue ? pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true, true>, grid, block, 0, stream, k)
                      : pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false, true>, grid, block, 0, stream, k);
+  }
+  if constexpr (NT == 1 && W == 1 && KVT == PA_DTYPE_FP8_E4M3FN) {
+    if (c.team)
+      return pa_launch(pa_partition_kernel<1, KVT, PT, BS16, 1, OCC, false, false, true>, grid, dim3(64 * kTeamWaves), 0, stream, k);
   }
   if (c.queue) return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, true>, grid, block, 0, stream, k);
   return pa_launch(pa_partition_kernel<NT, KVT, PT, BS16, W, OCC, false>, grid, block, 0, stream, k);
@@ -578,7 +607,7 @@ int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
   const int rc = check_partition(a);
   if (rc) return rc;
   if (generic_head_size(*a)) return launch_partition_generic(*a, reinterpret_cast<hipStream_t>(hip_stream));
-  return launch_partition(*a, choose_launch(*a), reinterpret_cast<hipStream_t>(hip_stream));
+  return launch_partition(*a, choose_launch(*a, false), reinterpret_cast<hipStream_t>(hip_stream));
 }
 
 int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
@@ -602,11 +631,12 @@ int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
     rc = launch_partition_generic(*a, reinterpret_cast<hipStream_t>(hip_stream));
     return rc ? rc : launch_reduce_generic(a, hip_stream);
   }
-  const LaunchChoice c = choose_launch(*a);
+  const LaunchChoice c = choose_launch(*a, true);
   rc = launch_partition(*a, c, reinterpret_cast<hipStream_t>(hip_stream));
   if (rc) return rc;
   // the partition kernel has written the rows of every sequence that has a single partition itself
   if (a->max_num_partitions == 1 && !a->sinks) return PA_OK;
+  if (c.team) return PA_OK;  // ... and a team those of every sequence
   if (c.listed_reduce) return launch_reduce_listed(a, hip_stream);
   return launch_reduce(a, hip_stream, true);
 }
@@ -620,7 +650,7 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
              a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? "fp8" : "bf16", generic_partition_blocks(*a));
     return PA_OK;
   }
-  const LaunchChoice c = choose_launch(*a);
+  const LaunchChoice c = choose_launch(*a, a->output != nullptr);  // (pa_decode's launch; pa_decode_partition forms no teams)
   const char* cache = !c.fp8 ? "bf16" : (c.per_token ? "fp8 per-token" : "fp8");
   const char* placed = c.heads_share_xcd ? ", an item's heads on one XCD" : "";
   if (c.shared)
@@ -629,8 +659,11 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
              placed);
   else
   {
-    char span_text[48] = "";
-    if (c.span > 1) snprintf(span_text, sizeof(span_text), ", %d partitions per workgroup", c.span);
+    char span_text[96] = "";
+    if (c.team)
+      snprintf(span_text, sizeof(span_text), ", teams of %d waves, %d partitions per wave, no reduce kernel", kTeamWaves, c.span);
+    else if (c.span > 1)
+      snprintf(span_text, sizeof(span_text), ", %d partitions per workgroup", c.span);
     snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s%s%s", cache,
              c.bs16 ? "bs16" : "strided", c.waves, c.row_tiles == 2 ? ", 2 row tiles" : "", c.blocks,
              c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""), span_text, placed);

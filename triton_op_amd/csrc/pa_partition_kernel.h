@@ -58,9 +58,15 @@ constexpr int kQueueMaxSeqs = 2048;  // sequences the item table of the queued l
 // REREAD: the kv head has more row tiles than a workgroup takes (a bf16 cache with more than 32 query rows), so a
 // second workgroup streams the same pages at about the same time: the cache is then read with ordinary loads (the
 // lines had better still be in L2 when the other workgroup asks; non-temporal loads mark them for early eviction).
-template <int NT, int KVT, bool PER_TOKEN, bool BS16, int WAVES, int OCC, bool QUEUE, bool REREAD = false>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+// TEAM (with WAVES = 1): four one-wave span walkers in ONE workgroup, wave w walking partitions w * span .. of the
+// same (sequence, kv head, row tile), each exactly as a one-wave workgroup would.  When the four spans cover the
+// whole partition axis, every partial result of the sequence is in this workgroup's LDS at the end, and the
+// workgroup merges them into `output` itself: no second kernel (a caller's fixed 256-token partitions over a 4096-
+// token context: 6 us of a 95 us call).
+template <int NT, int KVT, bool PER_TOKEN, bool BS16, int WAVES, int OCC, bool QUEUE, bool REREAD = false, bool TEAM = false>
+__global__ __launch_bounds__(TEAM ? 256 : 64 * WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 void pa_partition_kernel(const PaDecodeArgs a) {
+  static_assert(!TEAM || (WAVES == 1 && !QUEUE && NT == 1), "a team is four one-wave span walkers of one row tile");
   constexpr bool kFp8 = KVT == PA_DTYPE_FP8_E4M3FN;
   constexpr bool FP8MATH = kFp8;  // an FP8 cache is multiplied on the FP8 MFMAs, a bf16 cache on the bf16 ones
   constexpr int esz = kFp8 ? 1 : 2;
@@ -73,10 +79,12 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   // tile has no more real rows than that: half the bytes, twice the partitions), then 16 maxima and 16 sums.
   constexpr bool kSpanCapable = WAVES == 1 && !QUEUE;
   __shared__ __attribute__((aligned(16))) char o_lds[1][kSpanCapable ? 16 : 16 * kORowBytes];
-  __shared__ __attribute__((aligned(16))) char span_lds[kSpanCapable ? NT * kSpanPoolBytes : 16];
+  __shared__ __attribute__((aligned(16))) char span_lds[kSpanCapable ? (TEAM ? kTeamWaves : 1) * NT * kSpanPoolBytes : 16];
 
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int team_wave = TEAM ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+  const int wave = TEAM ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  char* const span_pool = &span_lds[0] + (kSpanCapable ? team_wave * NT * kSpanPoolBytes : 0);  // this wave's staging pool
   const int li = lane & 15;
   const int kg = lane >> 4;
 
@@ -186,7 +194,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       h = (int)(unit % (uint32_t)Hkv);
       rt = (int)(unit / (uint32_t)Hkv);
       item = (slot / units) * 8u + xcd;
-      if (!(a.flags & kFlagSortedItems) && item >= (uint32_t)a.num_seqs * (uint32_t)((P + span - 1) / span)) return;
+      if (!(a.flags & kFlagSortedItems) && item >= (uint32_t)a.num_seqs * (uint32_t)(TEAM ? 1 : (P + span - 1) / span)) return;
     } else {
       h = (int)(wid % (uint32_t)Hkv);
       rt = (int)((wid / (uint32_t)Hkv) % (uint32_t)RT);
@@ -208,7 +216,12 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     }
   }
   const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
+  const int team_part0 = part;     // TEAM: the workgroup's first partition (0: a team takes the whole axis)
+  if constexpr (TEAM) part += team_wave * span;
   do {  // the body of one item; `break` leaves it
+  if constexpr (TEAM) {
+    if (part >= P) break;  // (a wave of the team with no partition left)
+  }
 
   // The block-table entries of this wave's first step are requested together with the context length, not after it
   // (dependent scalar loads are round trips under full memory load; the first request of a workgroup waits for
@@ -226,7 +239,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const int ctx = sload_i32(a.context_lens + b);
   const int wg_start = part * a.partition_size;
   if (wg_start >= ctx) {
-    if (ctx <= 0 && part == 0) {
+    if (ctx <= 0 && part == 0 && !TEAM) {
       if constexpr (QUEUE) {  // only tiles with real query rows are items: the first one zeroes the whole group
         if (rt == 0) zero_output_rows(a, b, h, 0, Ge);
       } else {
@@ -772,7 +785,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const float acc_unit = FP8MATH ? (PER_TOKEN ? v_run[nt] : 1.f) * (1.f / 256.f) : 1.f;
-          char* slot = &span_lds[0] + ((part_cur - part) * NT + nt) * span_slot_bytes;
+          char* slot = span_pool + ((part_cur - part) * NT + nt) * span_slot_bytes;
           float l_tot = quad_row_sum(l_run[nt]);
           float m_out = m_run[nt];
           if (row0 + 16 * nt + li >= rows_valid) {  // padding rows of a ragged batch: no visible key
@@ -841,9 +854,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const bool direct = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
   // PA_DECODE_FLAG_OUTPUT_ONLY: rows beyond the sequence's query length are nobody's, and a sequence finished here
-  // leaves no partition-buffer entries
+  // leaves no partition-buffer entries (nor does any sequence of a team: its merge reads the staging pools)
   const bool output_only = a.flags & kFlagOutputOnly;
-  const bool no_partial = output_only && direct;
+  const bool no_partial = output_only && (direct || TEAM);
   const int rows_live = output_only ? rows_valid : Ge;
   float l_tot[NT], acc_unit[NT];
 #pragma unroll
@@ -864,10 +877,19 @@ void pa_partition_kernel(const PaDecodeArgs a) {
         a.max_logits[es_off + row] = m_run[nt] * (1.0f / kLog2e);
         a.exp_sums[es_off + row] = l_tot[nt];
       }
+      if constexpr (TEAM) {  // (the team's merge reads every partition's maximum and sum from the staging pools)
+        if (kg == 0) {
+          float* ml = reinterpret_cast<float*>(span_pool + ((part_cur - part) * NT + nt) * span_slot_bytes + span_rows * kORowBytes);
+          ml[li] = m_run[nt] * (1.0f / kLog2e);
+          ml[16 + li] = l_tot[nt];
+        }
+      }
       // (one-wave workgroups stage the last partition's tile in the next free slot of the pool)
-      char* stage_at = kSpanCapable ? &span_lds[0] + ((part_cur - part) * NT + nt) * span_slot_bytes : &o_lds[0][0];
+      char* stage_at = kSpanCapable ? span_pool + ((part_cur - part) * NT + nt) * span_slot_bytes : &o_lds[0][0];
       char* out_tile = outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2;
-      if (no_partial)
+      if (no_partial && !direct)
+        stage_partial_tile(stage_at, acc[nt], inv, lane, span_rows);
+      else if (no_partial)
         store_partial_tile(stage_at, acc[nt], inv, out_tile, a.stride_out_h * 2, nullptr, 0, rows_live - row0 - 16 * nt,
                            lane, kSpanCapable ? span_rows : 16);
       else
@@ -940,13 +962,13 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   if constexpr (kSpanCapable) {
     // SPAN: the partitions left behind on the way (a sequence that crosses a boundary has more than one
     // partition: nothing of it goes to `output` directly)
-    for (int pc = part; pc < part_cur; ++pc) {
+    for (int pc = part; pc < part_cur && !no_partial; ++pc) {
       const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)pc * a.stride_es_p;
       char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                         (int64_t)pc * a.stride_tmp_p) * 2;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const char* slot = &span_lds[0] + ((pc - part) * NT + nt) * span_slot_bytes;
+        const char* slot = span_pool + ((pc - part) * NT + nt) * span_slot_bytes;
         const int row = row0 + 16 * nt + li;
         if (row < rows_live && kg == 0) {
           a.max_logits[eo + row] = reinterpret_cast<const float*>(slot + span_rows * kORowBytes)[li];
@@ -971,6 +993,94 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     }
   }
   } while (0);
+  if constexpr (TEAM) {
+    // ---- the team's merge: every partial result of the sequence is staged in this workgroup's LDS ---------------
+    // (the sequence's lengths again: a wave without a partition has not read them; asked for ahead of the barrier)
+    const int ctx_t = sload_i32(a.context_lens + b);
+    const int qb_t = a.q_lens ? sload_i32(a.q_lens + b) : a.q_len;
+    int n_live = (ctx_t + a.partition_size - 1) / a.partition_size;
+    n_live = n_live > P ? P : n_live;
+    __syncthreads();
+    const int rows_valid_t = n_live > 0 ? qb_t * a.group_size : 0;
+    const bool output_only_t = a.flags & kFlagOutputOnly;
+    // (a sequence of one partition got its rows from the wave that finished it; with attention sinks or without an
+    // output the launch layer does not form teams)
+    const bool finished = n_live == 1 && ctx_t > 0;
+    char* outp_t = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
+    if (!finished && team_part0 == 0) {
+      // A half-wave per row (lane: four head dims), two rows of the tile per wave and pass.  Every lane takes the
+      // row's maximum over the partitions, then adds up its four dims with the partitions' weights (the maxima and
+      // sums are LDS broadcasts: no lane exchanges, and the reads of an unrolled group are independent).
+      const int half = lane >> 5, hl = lane & 31;
+      const int rows_here = Ge - row0 < 16 ? Ge - row0 : 16;  // rows of this tile that the buffers hold
+      for (int r0 = 2 * team_wave; r0 < rows_here; r0 += 2 * kTeamWaves) {
+        const int r = r0 + half;
+        const bool in_buf = r < rows_here;
+        const bool live = in_buf && row0 + r < rows_valid_t;
+        const int r_read = in_buf ? r : r0;  // (a row the pools hold)
+        // (wave w2's partitions are the slots of pool w2, in order: no division by the run-time span)
+        // Straight-line groups of four partitions: the LDS reads of a group are all requested before the first is
+        // used (an index past the pool's last live slot is clamped and its weight set to zero).
+        float M = -INFINITY;
+        for (int w2 = 0, p0 = 0; w2 < kTeamWaves && p0 < n_live; ++w2, p0 += span) {
+          const int cnt = n_live - p0 < span ? n_live - p0 : span;
+          const char* ml0 = &span_lds[0] + w2 * (NT * kSpanPoolBytes) + span_rows * kORowBytes + r_read * 4;
+          for (int j2 = 0; j2 < cnt; j2 += 4) {
+            float mp[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int jj = j2 + u < cnt ? j2 + u : cnt - 1;
+              mp[u] = *reinterpret_cast<const float*>(ml0 + jj * span_slot_bytes);
+            }
+            M = fmaxf(fmaxf(M, fmaxf(mp[0], mp[1])), fmaxf(mp[2], mp[3]));
+          }
+        }
+        const float M_safe = M == -INFINITY ? 0.f : M;
+        float L = 0.f;
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int w2 = 0, p0 = 0; w2 < kTeamWaves && p0 < n_live; ++w2, p0 += span) {
+          const int cnt = n_live - p0 < span ? n_live - p0 : span;
+          const char* pool = &span_lds[0] + w2 * (NT * kSpanPoolBytes);
+          for (int j2 = 0; j2 < cnt; j2 += 4) {
+            float lp[4], mp[4];
+            u32x2 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int jj = j2 + u < cnt ? j2 + u : cnt - 1;
+              const char* slot = pool + jj * span_slot_bytes;
+              const float* ml = reinterpret_cast<const float*>(slot + span_rows * kORowBytes);
+              lp[u] = ml[16 + r_read];
+              mp[u] = ml[r_read];
+              v[u] = *reinterpret_cast<const u32x2*>(slot + r_read * kORowBytes + hl * 8);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              // (a sum of zero comes with a maximum of -inf: weight zero; such a partition's rows may hold anything)
+              float wp = lp[u] * __expf(mp[u] - M_safe);
+              wp = j2 + u < cnt ? wp : 0.f;
+              const uint32_t keep = wp != 0.f ? 0xffffffffu : 0u;
+              const uint32_t v0 = v[u][0] & keep, v1 = v[u][1] & keep;
+              L += wp;
+              o[0] = fmaf(wp, bf16_bits_to_f32(v0 & 0xffffu), o[0]);
+              o[1] = fmaf(wp, __uint_as_float(v0 & 0xffff0000u), o[1]);
+              o[2] = fmaf(wp, bf16_bits_to_f32(v1 & 0xffffu), o[2]);
+              o[3] = fmaf(wp, __uint_as_float(v1 & 0xffff0000u), o[3]);
+            }
+          }
+        }
+        const float inv = L > 0.f ? 1.f / L : 0.f;
+#pragma unroll
+        for (int i2 = 0; i2 < 4; ++i2) o[i2] *= inv;
+        if (in_buf) {
+          u32x2* dst = reinterpret_cast<u32x2*>(outp_t + (int64_t)(row0 + r) * a.stride_out_h * 2 + hl * 8);
+          if (live)
+            *dst = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+          else if (!output_only_t || n_live <= 0)
+            *dst = u32x2{0u, 0u};  // padding rows (and every row of an empty sequence) read as zero
+        }
+      }
+    }
+  }
   if constexpr (!QUEUE) break;
   }  // for (;;)
   if constexpr (QUEUE) {
