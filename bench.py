@@ -283,6 +283,9 @@ def _time_config(lib, cfg, stream, steps, warmup, settle):
     # (a launch in teams merges in the partition kernel: pa_decode is that one kernel, pa_decode_partition another launch)
     team = "no reduce kernel" in cfg.launch
     solo = plans[0].args.max_num_partitions == 1 or team
+    if "own partitions of " in cfg.launch:  # (output-only: the library's own cut of the partition axis; one partition?)
+        own = int(cfg.launch.split("own partitions of ")[1].split()[0])
+        solo = solo or own >= plans[0].args.max_num_partitions * plans[0].args.partition_size
     r_us_avg = None
     if solo:
         k_launches = max(steps, 100)  # (a short run's 20 launches would mostly measure the first one's ramp)
@@ -540,7 +543,11 @@ def _bench_decode(a) -> int:
         # c2 at the configuration's literal partition size 256 (the reference's constant): same pools
         c2_256 = _Config("c2", dev, a.pools, 256, shared_from=cfg)
         lines.append(_config_line(c2_256, _time_config(lib, c2_256, stream, min(a.steps, 30), 5, a.settle)))
-        del c2_256
+        # ... and the same reference-shaped buffers as scratch (PA_DECODE_FLAG_OUTPUT_ONLY): the library cuts the
+        # partition axis its own way inside them
+        c2_256_lean = _Config("c2", dev, a.pools, 256, shared_from=c2_256, output_only=True)
+        lines.append(_config_line(c2_256_lean, _time_config(lib, c2_256_lean, stream, min(a.steps, 30), 5, a.settle)))
+        del c2_256, c2_256_lean
         for name in ("c3", "c4", "c5"):
             other = _Config(name, dev, 1)  # each of them streams far more than the last-level cache holds
             lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 30), 5, a.settle)))
@@ -549,7 +556,9 @@ def _bench_decode(a) -> int:
                 # which is what the configuration is there to stress
                 c4_256 = _Config("c4", dev, 1, 256, shared_from=other)
                 lines.append(_config_line(c4_256, _time_config(lib, c4_256, stream, min(a.steps, 30), 5, a.settle)))
-                del c4_256
+                c4_256_lean = _Config("c4", dev, 1, 256, shared_from=c4_256, output_only=True)
+                lines.append(_config_line(c4_256_lean, _time_config(lib, c4_256_lean, stream, min(a.steps, 30), 5, a.settle)))
+                del c4_256, c4_256_lean
             if name == "c5":
                 # ... and as an engine calls it that reads only the real query rows of `output`: no partition-buffer
                 # entries for the sequences stage 1 finishes, no zeros for the rows beyond a sequence's query length

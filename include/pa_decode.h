@@ -53,6 +53,14 @@ extern "C" {
  * beyond a sequence's own query length are left as they were instead of being zeroed.  Writes cost this GPU about
  * three times what reads cost: on a ragged batch of 256 sequences with 1-4 new tokens in buffers padded to 4
  * (70 MB of partial results, zeros and outputs per call) this is 6 % of the call.
+ * Scratch buffers also leave the cut of the partition axis to the library: a caller whose buffers are laid out for a
+ * small fixed partition_size (the reference's 256) gets fewer, longer partitions inside the same buffers -- the
+ * largest multiple of partition_size that is not above the tuning layer's own choice for the shape
+ * (pa_decode_launch_info says "own partitions of N tokens"; 64 sequences x 8 kv heads x 4096 tokens at 256: 89-91 ->
+ * 83 us).  Contexts are still cut off at max_num_partitions * partition_size tokens and no block-table entry beyond
+ * that token is read; when the factor does not divide max_num_partitions this needs a workspace of
+ * pa_decode_workspace_bytes (a limited copy of context_lens is kept there; without one the factor is the largest
+ * divisor), and a sequence that IS cut off counts the causal offsets of its new tokens from the cut.
  */
 #define PA_DECODE_FLAG_OUTPUT_ONLY 2
 
@@ -224,8 +232,8 @@ int pa_decode(const PaDecodeArgs* args, void* hip_stream);
  *
  * Environment: none of the library's behaviour depends on environment variables unless the process was started
  * with PA_DECODE_DEBUG=1, which enables the tuning switches PA_DECODE_WAVES, PA_DECODE_ROW_TILES, PA_DECODE_SPAN,
- * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED, PA_DECODE_LDS_PAD, PA_DECODE_P_RESIDUAL, PA_DECODE_XCD and
- * PA_DECODE_TEAM (read once, at the first launch).
+ * PA_DECODE_QUEUE, PA_DECODE_SHARED, PA_DECODE_SORTED, PA_DECODE_LDS_PAD, PA_DECODE_P_RESIDUAL, PA_DECODE_XCD,
+ * PA_DECODE_TEAM and PA_DECODE_REPARTITION (read once, at the first launch).
  */
 int pa_decode_launch_info(const PaDecodeArgs* args, char* text, int32_t text_bytes);
 

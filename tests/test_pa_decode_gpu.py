@@ -495,7 +495,8 @@ def test_teams_merge_in_the_partition_kernel(cuda, scale_mode, group, q_len, rag
     results into `output` themselves; pa_decode launches no reduce kernel (the launch layer says so).  Contexts end
     on, before and after partition and walk boundaries, reach one partition only (written by the wave that finished
     them), leave whole waves of a team without a partition, or are empty (zero rows).  The partition buffers are
-    held against the oracle's partition stage (with the output-only flag they are scratch and stay untouched), the
+    held against the oracle's partition stage (with the output-only flag the library cuts the partition axis its own
+    way -- one partition for these shapes, no teams -- and the same rows are checked), the
     result against the oracle; a second call with the same arguments is bit-identical.  With attention sinks no teams
     are formed."""
     import triton_op_amd as T
@@ -524,7 +525,10 @@ def test_teams_merge_in_the_partition_kernel(cuda, scale_mode, group, q_len, rag
     P = -(-max_ctx // ps)
     assert plan.args.max_num_partitions == P
     info = plan.launch_info()
-    assert f"teams of 4 waves, {per_wave} partitions per wave, no reduce kernel" in info and f"x {batch * 8}," in info, info
+    if output_only:  # the partition buffers are scratch: the library cuts the axis its own way (here: one partition)
+        assert "teams" not in info and "own partitions of" in info, info
+    else:
+        assert f"teams of 4 waves, {per_wave} partitions per wave, no reduce kernel" in info and f"x {batch * 8}," in info, info
     plan.exp_sums.fill_(float("nan"))
     plan.max_logits.fill_(float("nan"))
     plan.tmp_output.fill_(float("nan"))
@@ -533,9 +537,7 @@ def test_teams_merge_in_the_partition_kernel(cuda, scale_mode, group, q_len, rag
     first = out.clone()
     rows = (torch.ones(batch, dtype=torch.int32) * q_len if q_lens is None else q_lens)
     gml, ges, gto = plan.max_logits.cpu(), plan.exp_sums.cpu(), plan.tmp_output.float().cpu()
-    if output_only:
-        assert torch.isnan(gml).all() and torch.isnan(ges).all() and torch.isnan(gto).all()
-    else:
+    if not output_only:
         reach = (torch.arange(P)[None, :] * ps < ctx[:, None])  # [batch, P]
         ml, es, to = O.partition_stage(
             wl.query, wl.key_cache, wl.value_cache, wl.context_lens, wl.block_tables, wl.softmax_scale,
@@ -576,7 +578,8 @@ def test_teams_merge_in_the_partition_kernel(cuda, scale_mode, group, q_len, rag
     got2 = by_pos(out2)
     for b in live:
         n = int(rows[b])
-        torch.testing.assert_close(got2[b, :, :n], got[b, :, :n], atol=2e-3, rtol=2e-2)
+        # (with the output-only flag `got` comes from one long partition: no bf16 rounding of partial results)
+        torch.testing.assert_close(got2[b, :, :n], got[b, :, :n], atol=ATOL if output_only else 2e-3, rtol=2e-2)
 
 
 @pytest.mark.parametrize("seed", range(12))
@@ -1074,8 +1077,9 @@ def test_heads_of_an_item_on_one_xcd_in_plain_order(cuda, num_q_heads, q_len, ba
 @pytest.mark.parametrize("partition_size", [256, 1024, 4096])
 @pytest.mark.parametrize("with_sinks", [False, True])
 def test_output_only_flag(cuda, pa_lib, name, partition_size, with_sinks):
-    """PA_DECODE_FLAG_OUTPUT_ONLY: the caller reads only the real query rows of `output`.  Those rows equal the
-    flagless call's bit for bit (and so the oracle's, which that call is tested against); rows beyond a sequence's
+    """PA_DECODE_FLAG_OUTPUT_ONLY: the caller reads only the real query rows of `output`.  Those rows equal, bit for
+    bit, the flagless call's at the partition size the library cuts the axis into under the flag (a multiple of the
+    caller's; `pa_decode_launch_info` names it), and so the oracle's, which that call is tested against; rows beyond a sequence's
     query length are never NaN-poisoned into real rows; a sequence that stage 1 finishes leaves its padding rows as
     they were and its partition-buffer entries untouched; the two stage entry points called one by one with the flag
     give the same rows as pa_decode."""
@@ -1093,12 +1097,19 @@ def test_output_only_flag(cuda, pa_lib, name, partition_size, with_sinks):
                              g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
                              partition_size=partition_size, query_lens=g.q_lens, sinks=sinks, **kw)
 
-    ref = torch.full_like(g.query, float("nan"))
-    plan(ref).run()
     out = torch.full_like(g.query, 7.0)
     p = plan(out, output_only=True)
     p.exp_sums.fill_(-3.0)
     p.run()
+    # with the flag the library may cut the partition axis into fewer, longer partitions (the launch says so): the
+    # flagless call to compare with is the one at that partition size
+    info = p.launch_info()
+    own_size = int(info.split("own partitions of ")[1].split()[0]) if "own partitions of" in info else partition_size
+    assert own_size % partition_size == 0, info
+    ref = torch.full_like(g.query, float("nan"))
+    T.plan_decode(ref, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                  g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
+                  partition_size=own_size, query_lens=g.q_lens, sinks=sinks).run()
     two = torch.full_like(g.query, 7.0)
     p2 = plan(two, output_only=True)
     p2.run_partition()
@@ -1115,6 +1126,65 @@ def test_output_only_flag(cuda, pa_lib, name, partition_size, with_sinks):
         if finished_by_stage_1 and ctx > 0:
             assert torch.all(view(out)[b, :, ql:] == 7.0), f"padding rows of sequence {b} were written"
             assert torch.all(p.exp_sums[b] == -3.0), f"partition-buffer entries of sequence {b} were written"
+
+
+@pytest.mark.parametrize("batch,hkv,group,q_len,P,scale_mode,own",
+                         [(16, 2, 8, 1, 13, "tensor", 512), (24, 8, 8, 1, 29, "tensor", 2560),
+                          (40, 4, 8, 4, 29, "token", 1536), (12, 8, 16, 4, 13, "token", 768)])
+def test_output_only_cut_that_does_not_divide_the_partition_count(cuda, batch, hkv, group, q_len, P, scale_mode, own):
+    """PA_DECODE_FLAG_OUTPUT_ONLY with reference-shaped buffers (256-token partitions) whose partition count is a
+    prime: the library's own, longer partitions do not end where the caller's axis ends, so the kernels get the
+    context lengths with the caller's limit applied (a copy in the workspace).  One sequence's true context is
+    longer than the stated maximum: it is cut off at the end of the caller's axis, as without the flag (compared with
+    the oracle on the cut context when there is one new token; with several, the causal offsets of a cut-off sequence
+    count from the cut, and it is only checked to be finite).  The stage entry points called one by one give the
+    same bits; without a workspace the cut falls back to a divisor of the partition count (none for a prime: the
+    caller's partitions), with the same rows to the parity tolerance."""
+    import triton_op_amd as T
+
+    ps, axis = 256, 256 * P
+    gen = torch.Generator().manual_seed(4242 + P + batch)
+    ctx = torch.randint(1, axis + 1, (batch,), generator=gen, dtype=torch.int32)
+    ctx[0], ctx[1], ctx[2] = axis, 1, axis + 300  # (the third: longer than the stated maximum)
+    ctx = torch.clamp(ctx, min=q_len)
+    q_lens = torch.randint(1, q_len + 1, (batch,), generator=gen, dtype=torch.int32) if q_len > 1 else None
+    wl = _make(batch=batch, num_q_heads=group * hkv, num_kv_heads=hkv, context_lens=ctx, q_len=q_len, q_lens=q_lens,
+               kv_dtype="fp8", scale_mode=scale_mode, block_size=16, seed=4242 + P)
+    g = wl.to(cuda)
+
+    def plan(out, **kw):
+        return T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
+                             q_len, axis, torch.bfloat16, None, g.key_scale, g.value_scale, partition_size=ps,
+                             query_lens=g.q_lens, output_only=True, **kw)
+
+    out = torch.full_like(g.query, 7.0)
+    p = plan(out)
+    assert p.args.max_num_partitions == P
+    assert f"own partitions of {own} tokens" in p.launch_info() and P % (own // ps) != 0, p.launch_info()
+    p.run()
+    two = torch.full_like(g.query, 7.0)
+    p2 = plan(two)
+    p2.run_partition()
+    p2.run_reduce()
+    bare = torch.full_like(g.query, 7.0)
+    p3 = plan(bare)
+    p3.args.workspace = None
+    p3.args.workspace_bytes = 0
+    assert "own partitions" not in p3.launch_info(), p3.launch_info()
+    p3.run()
+    torch.cuda.synchronize()
+    by_pos = lambda t: t.float().cpu().view(batch, hkv, q_len, group, -1)
+    cut = type(wl)(**{**wl.__dict__, "context_lens": torch.clamp(ctx, max=axis)})
+    want = by_pos(_oracle(cut))
+    got, got2, got3 = by_pos(out), by_pos(two), by_pos(bare)
+    for b in range(batch):
+        n = q_len if q_lens is None else int(q_lens[b])
+        assert torch.equal(got[b, :, :n], got2[b, :, :n]), b
+        assert torch.isfinite(got[b, :, :n]).all() and torch.isfinite(got3[b, :, :n]).all(), b
+        if b == 2 and q_len > 1:
+            continue
+        torch.testing.assert_close(got[b, :, :n], want[b, :, :n], atol=ATOL, rtol=RTOL)
+        torch.testing.assert_close(got3[b, :, :n], want[b, :, :n], atol=ATOL, rtol=RTOL)
 
 
 def _random_case_wide(seed):

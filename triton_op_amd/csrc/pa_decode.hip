@@ -12,6 +12,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include <mutex>
 
@@ -32,6 +33,12 @@ static __device__ __align__(256) unsigned char scratch[PA_DECODE_NOALLOC_SCRATCH
 thread_local int pa_last_hip_error = 0;
 
 namespace {
+
+// context lengths with a limit applied (the end of a caller's partition axis)
+__global__ void pa_limit_lens_kernel(const int32_t* lens, int32_t* out, int n, int limit) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = lens[i] < limit ? lens[i] : limit;
+}
 
 // the first `n` int32 words at p become zero (a launch, not a memset node: callers may be capturing a graph)
 __global__ void pa_clear_words_kernel(int32_t* p, int n) {
@@ -603,18 +610,80 @@ int pa_decode_select_partition_size_stats(int32_t num_seqs_given, int32_t num_kv
   }
 }
 
-int pa_decode_partition(const PaDecodeArgs* a, void* hip_stream) {
-  const int rc = check_partition(a);
+// PA_DECODE_FLAG_OUTPUT_ONLY: the partition buffers are scratch, so how the partition axis is cut is the library's
+// business.  A caller's small fixed partition size (the reference's constant 256) is replaced by the largest multiple
+// of it that is not above the tuning layer's own choice for the shape: fewer, longer partitions, every entry of which
+// lies inside the caller's buffers, at the caller's strides.  The axis must still end where the caller's ends
+// (contexts beyond it are cut off at the same token, and no block-table entry beyond it is read).  With a factor that
+// divides the caller's partition count it does; with another factor the last partition reaches further, and the
+// kernels are then given a copy of the context lengths with the caller's limit applied (made by a small kernel, in
+// the caller's workspace behind the item list; without a workspace of pa_decode_workspace_bytes the factor is the
+// largest divisor).  The three entry points derive the same cut from the same arguments; `stream` is null when
+// nothing may be launched (pa_decode_launch_info).  PA_DECODE_REPARTITION=0 (debug): never.
+struct OwnPartitions {
+  PaDecodeArgs args;
+  int rc;
+};
+
+static OwnPartitions with_own_partitions(const PaDecodeArgs& a, bool launch, hipStream_t stream) {
+  OwnPartitions r{a, PA_OK};
+  static const bool off = debug_switch("PA_DECODE_REPARTITION", 1) == 0;
+  if (off || !(a.flags & PA_DECODE_FLAG_OUTPUT_ONLY) || a.max_num_partitions <= 1 || generic_head_size(a)) return r;
+  const long long axis = (long long)a.max_num_partitions * a.partition_size;
+  if (axis > 0x7fffffffLL) return r;
+  const int want = pa_decode_select_partition_size_stats(a.num_seqs, a.num_kv_heads, a.q_len * a.group_size, (int)axis, 0,
+                                                         a.block_size, 0);
+  const int P = a.max_num_partitions;
+  long long k = want / a.partition_size;
+  k = k > P ? P : k;
+  if (k < 2) return r;
+  if (P % k) {
+    const long long parts = (P + k - 1) / k;
+    // words of the workspace: header, item list of the new cut, [the limited lengths], ..., list of the sequences to merge
+    const long long first = kPlanHeaderWords + 2LL * a.num_seqs * parts;
+    const bool room = a.workspace != nullptr && a.workspace_bytes >= full_workspace_bytes(a.num_seqs, P) &&
+                      first + 2LL * a.num_seqs <= a.workspace_bytes / 4;
+    if (room) {
+      r.args.context_lens = a.workspace + first;
+      if (launch && !(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST))
+        r.rc = pa_launch(pa_limit_lens_kernel, dim3((unsigned)((a.num_seqs + 255) / 256)), dim3(256), 0, stream,
+                         a.context_lens, a.workspace + first, (int)a.num_seqs, (int)axis);
+    } else {
+      while (P % k) --k;  // the largest divisor below
+      if (k < 2) return r;
+    }
+  }
+  r.args.partition_size = (int32_t)(a.partition_size * k);
+  r.args.max_num_partitions = (int32_t)((P + k - 1) / k);
+  return r;
+}
+
+int pa_decode_partition(const PaDecodeArgs* caller, void* hip_stream) {
+  const int rc = check_partition(caller);
   if (rc) return rc;
+  const OwnPartitions own = with_own_partitions(*caller, true, reinterpret_cast<hipStream_t>(hip_stream));
+  if (own.rc) return own.rc;
+  const PaDecodeArgs* a = &own.args;
   if (generic_head_size(*a)) return launch_partition_generic(*a, reinterpret_cast<hipStream_t>(hip_stream));
   return launch_partition(*a, choose_launch(*a, false), reinterpret_cast<hipStream_t>(hip_stream));
 }
 
-int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
-  // PA_DECODE_FLAG_OUTPUT_ONLY: stage 1 ran with the same flag and left no entries for the sequences it finished
-  // itself; stage 2 passes over them, as it does inside pa_decode
-  if (a && a->struct_size == sizeof(PaDecodeArgs) && generic_head_size(*a)) return launch_reduce_generic(a, hip_stream);
-  const bool lean = a && a->struct_size == sizeof(PaDecodeArgs) && (a->flags & PA_DECODE_FLAG_OUTPUT_ONLY);
+int pa_decode_reduce(const PaDecodeArgs* caller, void* hip_stream) {
+  // PA_DECODE_FLAG_OUTPUT_ONLY: stage 1 ran with the same flag, cut the partition axis as with_own_partitions cuts
+  // it and left no entries for the sequences it finished itself; stage 2 passes over them, as it does inside pa_decode
+  if (caller && caller->struct_size == sizeof(PaDecodeArgs) && generic_head_size(*caller))
+    return launch_reduce_generic(caller, hip_stream);
+  const bool lean = caller && caller->struct_size == sizeof(PaDecodeArgs) && (caller->flags & PA_DECODE_FLAG_OUTPUT_ONLY);
+  OwnPartitions own;
+  const PaDecodeArgs* a = caller;
+  if (lean) {
+    const int rc = check_reduce(caller);  // (before the arguments are used)
+    if (rc) return rc;
+    // (the limited context lengths are made again: stage 2 does not rely on what stage 1 left in the workspace)
+    own = with_own_partitions(*caller, true, reinterpret_cast<hipStream_t>(hip_stream));
+    if (own.rc) return own.rc;
+    a = &own.args;
+  }
   if (lean && a->max_num_partitions == 1 && !a->sinks) {
     const int rc = check_reduce(a);
     return rc;  // every sequence was finished by stage 1
@@ -622,11 +691,14 @@ int pa_decode_reduce(const PaDecodeArgs* a, void* hip_stream) {
   return launch_reduce(a, hip_stream, lean);
 }
 
-int pa_decode(const PaDecodeArgs* a, void* hip_stream) {
-  int rc = check_partition(a);
+int pa_decode(const PaDecodeArgs* caller, void* hip_stream) {
+  int rc = check_partition(caller);
   if (rc) return rc;
-  rc = check_reduce(a);  // before anything is launched
+  rc = check_reduce(caller);  // before anything is launched
   if (rc) return rc;
+  const OwnPartitions own = with_own_partitions(*caller, true, reinterpret_cast<hipStream_t>(hip_stream));
+  if (own.rc) return own.rc;
+  const PaDecodeArgs* a = &own.args;
   if (generic_head_size(*a)) {
     rc = launch_partition_generic(*a, reinterpret_cast<hipStream_t>(hip_stream));
     return rc ? rc : launch_reduce_generic(a, hip_stream);
@@ -650,6 +722,9 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
              a->kv_dtype == PA_DTYPE_FP8_E4M3FN ? "fp8" : "bf16", generic_partition_blocks(*a));
     return PA_OK;
   }
+  const OwnPartitions own = with_own_partitions(*a, false, nullptr);
+  const bool recut = own.args.partition_size != a->partition_size;
+  a = &own.args;
   const LaunchChoice c = choose_launch(*a, a->output != nullptr);  // (pa_decode's launch; pa_decode_partition forms no teams)
   const char* cache = !c.fp8 ? "bf16" : (c.per_token ? "fp8 per-token" : "fp8");
   const char* placed = c.heads_share_xcd ? ", an item's heads on one XCD" : "";
@@ -667,6 +742,11 @@ int pa_decode_launch_info(const PaDecodeArgs* a, char* text, int32_t text_bytes)
     snprintf(text, (size_t)text_bytes, "pa_partition_kernel<%s, %s, %d waves%s> x %lld%s%s%s", cache,
              c.bs16 ? "bs16" : "strided", c.waves, c.row_tiles == 2 ? ", 2 row tiles" : "", c.blocks,
              c.queue ? ", queued items" : (c.sorted ? ", sorted items" : ""), span_text, placed);
+  }
+  if (recut) {  // PA_DECODE_FLAG_OUTPUT_ONLY: the library's own cut of the caller's partition axis
+    const size_t used = strlen(text);
+    if (used + 1 < (size_t)text_bytes)
+      snprintf(text + used, (size_t)text_bytes - used, ", own partitions of %d tokens", a->partition_size);
   }
   return PA_OK;
 }

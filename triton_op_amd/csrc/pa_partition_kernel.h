@@ -854,9 +854,9 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   const bool direct = (ctx <= a.partition_size || a.max_num_partitions == 1) && a.output != nullptr && a.sinks == nullptr;
   char* outp = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
   // PA_DECODE_FLAG_OUTPUT_ONLY: rows beyond the sequence's query length are nobody's, and a sequence finished here
-  // leaves no partition-buffer entries (nor does any sequence of a team: its merge reads the staging pools)
+  // leaves no partition-buffer entries
   const bool output_only = a.flags & kFlagOutputOnly;
-  const bool no_partial = output_only && (direct || TEAM);
+  const bool no_partial = output_only && direct;
   const int rows_live = output_only ? rows_valid : Ge;
   float l_tot[NT], acc_unit[NT];
 #pragma unroll
@@ -887,9 +887,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
       // (one-wave workgroups stage the last partition's tile in the next free slot of the pool)
       char* stage_at = kSpanCapable ? span_pool + ((part_cur - part) * NT + nt) * span_slot_bytes : &o_lds[0][0];
       char* out_tile = outp + (int64_t)(row0 + 16 * nt) * a.stride_out_h * 2;
-      if (no_partial && !direct)
-        stage_partial_tile(stage_at, acc[nt], inv, lane, span_rows);
-      else if (no_partial)
+      if (no_partial)
         store_partial_tile(stage_at, acc[nt], inv, out_tile, a.stride_out_h * 2, nullptr, 0, rows_live - row0 - 16 * nt,
                            lane, kSpanCapable ? span_rows : 16);
       else
@@ -962,7 +960,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
   if constexpr (kSpanCapable) {
     // SPAN: the partitions left behind on the way (a sequence that crosses a boundary has more than one
     // partition: nothing of it goes to `output` directly)
-    for (int pc = part; pc < part_cur && !no_partial; ++pc) {
+    for (int pc = part; pc < part_cur; ++pc) {
       const int64_t eo = (int64_t)b * a.stride_es_s + (int64_t)h * a.stride_es_h + (int64_t)pc * a.stride_es_p;
       char* tp = (char*)a.tmp_output + ((int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                                         (int64_t)pc * a.stride_tmp_p) * 2;

@@ -422,7 +422,9 @@ def paged_attention_decode(
     """Split-KV paged-attention decode; writes `output` in place on torch's current stream and
     returns the partition buffers under the reference's keys.  `output_only=True` (PA_DECODE_FLAG_OUTPUT_ONLY): the
     caller reads nothing but the rows of `output` that belong to real query rows; the partition buffers are scratch
-    with unspecified contents afterwards, and rows beyond a sequence's `query_lens` entry are left as they were."""
+    with unspecified contents afterwards, and rows beyond a sequence's `query_lens` entry are left as they were.
+    With a caller-fixed small `partition_size` the library then cuts the partition axis into fewer, longer partitions
+    of its own inside the same buffers (`plan.launch_info()` names their size)."""
     plan = plan_decode(
         output, query, key_cache, value_cache, sequence_lengths, block_tables, softmax_scale,
         query_sequence_length, max_sequence_length, compute_type, query_scale, key_scale, value_scale,
