@@ -38,7 +38,8 @@ extern "C" {
 #define PA_DECODE_WORKSPACE_BYTES 64
 /*
  * flags: the workspace still holds the item list that an earlier call built for the SAME context_lens contents,
- * num_seqs, num_kv_heads, q_len, group_size, block_size, max_num_partitions and partition_size (the previous layer
+ * num_seqs, num_kv_heads, q_len, group_size, block_size, max_num_partitions, partition_size and
+ * PA_DECODE_FLAG_OUTPUT_ONLY setting (the previous layer
  * of one decode step, say; the items a launch lists also depend on how many partitions it gives a workgroup, which
  * follows from those shapes): the planning kernel is skipped (about 4.5 us).  Ignored by launches that use no item
  * list.

@@ -645,7 +645,7 @@ static OwnPartitions with_own_partitions(const PaDecodeArgs& a, bool launch, hip
                       first + 2LL * a.num_seqs <= a.workspace_bytes / 4;
     if (room) {
       r.args.context_lens = a.workspace + first;
-      if (launch && !(a.flags & PA_DECODE_FLAG_REUSE_ITEM_LIST))
+      if (launch)  // (also when the item list is reused: 2 us, and the copy then never depends on an earlier call)
         r.rc = pa_launch(pa_limit_lens_kernel, dim3((unsigned)((a.num_seqs + 255) / 256)), dim3(256), 0, stream,
                          a.context_lens, a.workspace + first, (int)a.num_seqs, (int)axis);
     } else {
