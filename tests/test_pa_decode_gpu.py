@@ -720,13 +720,14 @@ def test_large_logits(cuda, name, gain):
     _check_stages(wl, res, 512)
 
 
-@pytest.mark.parametrize("case", ["queue", "sorted", "plain"])
+@pytest.mark.parametrize("case", ["queue", "sorted", "plain", "teams", "own_cut"])
 def test_graph_capture_and_replay(cuda, case):
     """A decode plan allocates nothing and only launches kernels on the given stream, so it can be captured
     in a HIP graph: every replay (with eager work and synchronisations in between, and with new inputs written
     into the captured tensors) must reproduce the eager result bit for bit.  Covers the launch modes that keep
     state in the workspace: the work queue (its counters return to zero) and the sorted dispatch (its list is
-    rebuilt by every call)."""
+    rebuilt by every call); a launch in teams; and the output-only flag with the library's own cut of a prime
+    partition count (the kernel that limits the context lengths is part of the graph)."""
     import triton_op_amd as T
 
     gen = torch.Generator().manual_seed(31)
@@ -738,6 +739,12 @@ def test_graph_capture_and_replay(cuda, case):
         # partitions each and 96 sequences would be a single round)
         kw = dict(batch=96, num_q_heads=128, num_kv_heads=8, q_len=2,
                   context_lens=torch.randint(2, 2600, (96,), generator=gen, dtype=torch.int32))
+    elif case == "teams":  # one workgroup per (sequence, kv head) that merges its partitions itself: a single kernel
+        kw = dict(batch=52, num_q_heads=64, num_kv_heads=8,
+                  context_lens=torch.randint(1, 2049, (52,), generator=gen, dtype=torch.int32))
+    elif case == "own_cut":  # output-only, a prime partition count: the limited context lengths are made inside the graph
+        kw = dict(batch=16, num_q_heads=16, num_kv_heads=2,
+                  context_lens=torch.cat([torch.randint(1, 3328, (15,), generator=gen, dtype=torch.int32), _ctx(3328)]))
     else:
         kw = dict(batch=3, num_q_heads=16, num_kv_heads=2, context_lens=_ctx(300, 64, 1000))
     wl = _make(**kw)
@@ -745,9 +752,10 @@ def test_graph_capture_and_replay(cuda, case):
     out = torch.full_like(g.query, float("nan"))
     plan = T.plan_decode(out, g.query, g.key_cache, g.value_cache, g.context_lens, g.block_tables, g.softmax_scale,
                          g.q_len, g.max_context_len, torch.bfloat16, None, g.key_scale, g.value_scale,
-                         partition_size=256, query_lens=g.q_lens)
+                         partition_size=256, query_lens=g.q_lens, output_only=case == "own_cut")
     if case != "plain":  # the launch mode the case is named for is the one that is captured
-        assert ("queued items" if case == "queue" else "sorted items") in plan.launch_info(), plan.launch_info()
+        mode = {"queue": "queued items", "sorted": "sorted items", "teams": "teams of 4 waves", "own_cut": "own partitions of 512 tokens"}
+        assert mode[case] in plan.launch_info(), plan.launch_info()
     plan.run()
     torch.cuda.synchronize()
     eager = out.clone()
