@@ -542,28 +542,28 @@ def _bench_decode(a) -> int:
         lines = []
         # c2 at the configuration's literal partition size 256 (the reference's constant): same pools
         c2_256 = _Config("c2", dev, a.pools, 256, shared_from=cfg)
-        lines.append(_config_line(c2_256, _time_config(lib, c2_256, stream, min(a.steps, 30), 5, a.settle)))
+        lines.append(_config_line(c2_256, _time_config(lib, c2_256, stream, min(a.steps, 100), 10, a.settle)))
         # ... and the same reference-shaped buffers as scratch (PA_DECODE_FLAG_OUTPUT_ONLY): the library cuts the
         # partition axis its own way inside them
         c2_256_lean = _Config("c2", dev, a.pools, 256, shared_from=c2_256, output_only=True)
-        lines.append(_config_line(c2_256_lean, _time_config(lib, c2_256_lean, stream, min(a.steps, 30), 5, a.settle)))
+        lines.append(_config_line(c2_256_lean, _time_config(lib, c2_256_lean, stream, min(a.steps, 100), 10, a.settle)))
         del c2_256, c2_256_lean
         for name in ("c3", "c4", "c5"):
             other = _Config(name, dev, 1)  # each of them streams far more than the last-level cache holds
-            lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 30), 5, a.settle)))
+            lines.append(_config_line(other, _time_config(lib, other, stream, min(a.steps, 100), 10, a.settle)))
             if name == "c4":
                 # ... and at the configuration's literal partition size: 512 partitions per sequence, the merge of
                 # which is what the configuration is there to stress
                 c4_256 = _Config("c4", dev, 1, 256, shared_from=other)
-                lines.append(_config_line(c4_256, _time_config(lib, c4_256, stream, min(a.steps, 30), 5, a.settle)))
+                lines.append(_config_line(c4_256, _time_config(lib, c4_256, stream, min(a.steps, 100), 10, a.settle)))
                 c4_256_lean = _Config("c4", dev, 1, 256, shared_from=c4_256, output_only=True)
-                lines.append(_config_line(c4_256_lean, _time_config(lib, c4_256_lean, stream, min(a.steps, 30), 5, a.settle)))
+                lines.append(_config_line(c4_256_lean, _time_config(lib, c4_256_lean, stream, min(a.steps, 100), 10, a.settle)))
                 del c4_256, c4_256_lean
             if name == "c5":
                 # ... and as an engine calls it that reads only the real query rows of `output`: no partition-buffer
                 # entries for the sequences stage 1 finishes, no zeros for the rows beyond a sequence's query length
                 c5_lean = _Config("c5", dev, 1, shared_from=other, output_only=True)
-                lines.append(_config_line(c5_lean, _time_config(lib, c5_lean, stream, min(a.steps, 30), 5, a.settle)))
+                lines.append(_config_line(c5_lean, _time_config(lib, c5_lean, stream, min(a.steps, 100), 10, a.settle)))
                 del c5_lean
             del other
             torch.cuda.empty_cache()
