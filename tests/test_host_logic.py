@@ -400,6 +400,46 @@ def _fake_args(*, b, hq, hkv, q, ctx, bs=16, ps, kv="fp8", per_token=False, ragg
     return a
 
 
+def test_own_cut_of_the_partition_axis_invariants(pa_lib):
+    """PA_DECODE_FLAG_OUTPUT_ONLY: over random shapes the library's own partition size (pa_decode_launch_info names
+    it) is a multiple of the caller's, no longer than the caller's whole axis and no longer than the tuning layer's
+    choice for the shape; without a workspace the factor divides the caller's partition count (the axis ends where
+    the caller's ends); without the flag nothing is re-cut."""
+    import random
+
+    rng = random.Random(77)
+    recut = 0
+    for _ in range(1500):
+        hkv = rng.choice([1, 2, 4, 8])
+        g, q = rng.choice([(1, 1), (5, 1), (8, 1), (16, 1), (8, 2), (16, 2), (16, 4), (8, 4), (10, 1)])
+        b = rng.choice([1, 3, 16, 64, 128, 256, 700])
+        ps = rng.choice([256, 256, 512, 1024])
+        ctx = rng.randint(1, 140000 if b <= 16 else 9000)
+        ws = rng.random() < 0.7
+        kw = dict(b=b, hq=g * hkv, hkv=hkv, q=q, ctx=ctx, bs=rng.choice([16, 64, 1024]), ps=ps,
+                  per_token=rng.random() < 0.5, ragged=q > 1 and rng.random() < 0.5, workspace=ws)
+        texts = []
+        for flags in (0, _cabi.PA_DECODE_FLAG_OUTPUT_ONLY):
+            a = _fake_args(**kw)
+            a.flags = flags
+            buf = C.create_string_buffer(256)
+            assert pa_lib.pa_decode_launch_info(C.byref(a), buf, 256) == 0, kw
+            texts.append(buf.value.decode())
+        assert "own partitions" not in texts[0], (kw, texts[0])
+        if "own partitions of " not in texts[1]:
+            continue
+        recut += 1
+        P = -(-ctx // ps)
+        own = int(texts[1].split("own partitions of ")[1].split()[0])
+        k = own // ps
+        assert own % ps == 0 and 2 <= k <= P, (kw, texts[1])
+        want = pa_lib.pa_decode_select_partition_size_stats(b, hkv, g * q, P * ps, 0, kw["bs"], 256)
+        assert own <= want, (kw, texts[1], want)
+        if not ws:
+            assert P % k == 0, (kw, texts[1])
+    assert recut > 300
+
+
 def test_launch_layer_choices(pa_lib):
     """Which partition kernel, in which instantiation, over which grid: the launch layer's choice for the five
     benchmark configurations at the tuning layer's partition size (256 compute units assumed when there is no
