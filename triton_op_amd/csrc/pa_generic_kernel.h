@@ -13,12 +13,17 @@ namespace {
 // on bf16 MFMAs without a software pipeline -- the same results, not the same speed.
 //
 // Stage 1: one wave per (sequence, partition, kv head, 16-row query tile).  A 64-token step is four 16-token
-// tiles.  v_mfma_f32_16x16x16_bf16 holds, in lane l (li = l % 16, kg = l / 16), four consecutive reduction indices
-// 4 kg .. 4 kg + 3 of row / column li of its operands and rows 4 kg .. 4 kg + 3 of column li of its result, so:
-//   S^T[token, row] = K Q^T:  A = 4 head dims of token li (a quarter of a 16-byte piece of the cache, as bf16),
+// blocks (pages, when the page size is 16).  v_mfma_f32_16x16x16_bf16 holds, in lane l (li = l % 16, kg = l / 16),
+// four consecutive reduction indices 4 kg .. 4 kg + 3 of row / column li of its operands and rows 4 kg .. 4 kg + 3 of
+// column li of its result, so:
+//   S^T[token, row] = K Q^T:  A = 4 head dims of a token (a quarter of a 16-byte piece of the cache, as bf16),
 //                             B = the same 4 head dims of query row li; the result holds 4 tokens of row li;
 //   O^T[dim, row]   = V^T P:  A = 4 tokens of head dim li of a 16-dim block, B = P of those 4 tokens for row li --
 //                             exactly what the lane holds of S^T, so P never moves between lanes.
+// Which token is row i of K tile j is free: tile j takes tokens 4 j .. 4 j + 3 of EVERY block (row i: block i / 4,
+// token 4 j + i % 4), so that lane group kg ends up with the logits, and then P, of all 16 tokens of block kg -- and
+// its V operands of the step's four MFMAs per 16-dim block are one 16-byte piece of the cache (16 tokens of head dim
+// li), not four 4-byte pieces of four blocks.
 // Row maximum and sum: 16 values in the lane, then the four lanes of a row (quad_row_max / quad_row_sum).
 // ---------------------------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(4))) short bf16x4_bits;
@@ -124,22 +129,39 @@ void pa_partition_generic_kernel(const PaDecodeArgs a) {
 #pragma unroll
   for (int db = 0; db < DB; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  const int sub_k = li >> 2;  // the 16-token block this lane's K rows come from (see the token order above)
+  // pages of a step's four 16-token blocks (blocks past the last live one repeat it); asked for one step ahead
+  int page_next[4];
+  auto load_pages = [&](int t0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int t = t0 + 16 * j;
+      t = t > last_tile_tok ? last_tile_tok : t;
+      page_next[j] = sload_i32(bt + (t >> log2_bs));
+    }
+  };
+  load_pages(wg_start);
   for (int tok0 = wg_start; tok0 < wg_end; tok0 += kStepTokens) {
-    // ---- pages of the step's four tiles (tiles past the last live one repeat it) ----------------------------------
     int page[4], off[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int t = tok0 + 16 * j;
       t = t > last_tile_tok ? last_tile_tok : t;
-      page[j] = sload_i32(bt + (t >> log2_bs));
+      page[j] = page_next[j];
       off[j] = t & bs_mask;
     }
-    // ---- S^T = K Q^T --------------------------------------------------------------------------------------------------
+    load_pages(tok0 + kStepTokens);  // (an index past the sequence's last live block is clamped to it)
+    // this lane's block as a row of K (li / 4) and as a holder of logits, P, scales and V (kg)
+    const int page_k = sub_k == 0 ? page[0] : (sub_k == 1 ? page[1] : (sub_k == 2 ? page[2] : page[3]));
+    const int off_k = (sub_k == 0 ? off[0] : (sub_k == 1 ? off[1] : (sub_k == 2 ? off[2] : off[3]))) + (li & 3);
+    const int page_v = kg == 0 ? page[0] : (kg == 1 ? page[1] : (kg == 2 ? page[2] : page[3]));
+    const int off_v = kg == 0 ? off[0] : (kg == 1 ? off[1] : (kg == 2 ? off[2] : off[3]));
+    // ---- S^T = K Q^T: tile j takes tokens 4 j .. 4 j + 3 of every block ---------------------------------------------
     f32x4 s[4];
+    const char* kt = kbase + (int64_t)page_k * a.stride_k_b * ESZ;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const char* kt = kbase + (int64_t)page[j] * a.stride_k_b * ESZ;
 #pragma unroll
       for (int g = 0; g < D / 64; ++g) {
         // this lane's 16 head dims of the 64-dim group: one 16-byte piece (FP8) or two (bf16)
@@ -148,10 +170,10 @@ void pa_partition_generic_kernel(const PaDecodeArgs a) {
           uint32_t u[8];
         } kv;
         if constexpr (FP8) {
-          kv.q[0] = load16(kt + (int64_t)(4 * g + kg) * a.stride_k_c + (off[j] + li) * 16);
+          kv.q[0] = load16(kt + (int64_t)(4 * g + kg) * a.stride_k_c + (off_k + 4 * j) * 16);
         } else {
-          kv.q[0] = load16(kt + ((int64_t)(8 * g + 2 * kg) * a.stride_k_c + (off[j] + li) * 8) * 2);
-          kv.q[1] = load16(kt + ((int64_t)(8 * g + 2 * kg + 1) * a.stride_k_c + (off[j] + li) * 8) * 2);
+          kv.q[0] = load16(kt + ((int64_t)(8 * g + 2 * kg) * a.stride_k_c + (off_k + 4 * j) * 8) * 2);
+          kv.q[1] = load16(kt + ((int64_t)(8 * g + 2 * kg + 1) * a.stride_k_c + (off_k + 4 * j) * 8) * 2);
         }
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
@@ -170,21 +192,22 @@ void pa_partition_generic_kernel(const PaDecodeArgs a) {
         }
       }
     }
-    // ---- scales, ALiBi, mask; row maximum ---------------------------------------------------------------------------
+    // ---- scales, ALiBi, mask; row maximum (s[j][r]: token 16 kg + 4 j + r of the step) ------------------------------
     f32x4 vs[4];
     float mx = -INFINITY;
+    const int col0 = tok0 + 16 * kg;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       f32x4 ks = {1.f, 1.f, 1.f, 1.f};
       vs[j] = f32x4{1.f, 1.f, 1.f, 1.f};
       if (per_token) {
-        const int64_t so = (int64_t)page[j] * a.stride_kvscale_b + (int64_t)h * a.stride_kvscale_h + off[j] + 4 * kg;
+        const int64_t so = (int64_t)page_v * a.stride_kvscale_b + (int64_t)h * a.stride_kvscale_h + off_v + 4 * j;
         ks = *reinterpret_cast<const f32x4*>(a.key_scale + so);
         vs[j] = *reinterpret_cast<const f32x4*>(a.value_scale + so);
       }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int col = tok0 + 16 * j + 4 * kg + r;
+        const int col = col0 + 4 * j + r;
         float x = s[j][r] * ks[r] * rscale + slope2 * (float)(col - ctx + 1);
         x = col < limit ? x : -INFINITY;  // (a select: stale cache bytes may have made the logit a NaN)
         s[j][r] = x;
@@ -218,25 +241,48 @@ void pa_partition_generic_kernel(const PaDecodeArgs a) {
     l_run = l_run * alpha + quad_row_sum(psum);
 #pragma unroll
     for (int db = 0; db < DB; ++db) acc[db] *= alpha;
-    // ---- O^T += V^T P -----------------------------------------------------------------------------------------------
+    // ---- O^T += V^T P: the lane's 16 tokens of head dim li are ONE 16-byte piece of the cache (two with bf16) ----------
+    // stale bytes past the context may decode to NaN, and 0 * NaN is NaN: those tokens' V is zero (masks per 4 tokens:
+    // FP8, one byte a token; bf16, two dwords of two tokens)
+    const int n_live = ctx - col0;  // live tokens of this lane's block (may be <= 0 or >= 16)
+    uint32_t keep[FP8 ? 4 : 8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int t4 = tok0 + 16 * j + 4 * kg;  // this lane's four tokens of the tile
-      const int o4 = off[j] + 4 * kg;
-      const char* vt = vbase + (int64_t)page[j] * a.stride_v_b * ESZ;
+    for (int w = 0; w < (FP8 ? 4 : 8); ++w) {
+      const int per = FP8 ? 4 : 2;  // tokens in dword w
+      const int v = n_live - per * w;
+      keep[w] = v >= per ? 0xffffffffu : (v <= 0 ? 0u : (FP8 ? (1u << (8 * v)) - 1u : 0xffffu));
+    }
+    const char* vt = vbase + (int64_t)page_v * a.stride_v_b * ESZ;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int d = 16 * db + li;
-        const int64_t e = a.v_transposed ? (int64_t)(o4 / X) * a.stride_v_2 + (int64_t)d * X + o4 % X
-                                         : (int64_t)d * a.stride_v_2 + o4;
+    for (int db = 0; db < DB; ++db) {
+      const int d = 16 * db + li;
+      union {
+        u32x4 q[2];
+        uint32_t u[8];
+      } vw;
+      if constexpr (FP8) {
+        const int64_t e = a.v_transposed ? (int64_t)(off_v / X) * a.stride_v_2 + (int64_t)d * X : (int64_t)d * a.stride_v_2 + off_v;
+        vw.q[0] = load16(vt + e);
+      } else {
+        const int64_t e0 = a.v_transposed ? (int64_t)(off_v / X) * a.stride_v_2 + (int64_t)d * X : (int64_t)d * a.stride_v_2 + off_v;
+        const int64_t e1 = a.v_transposed ? e0 + a.stride_v_2 : e0 + 8;
+        vw.q[0] = load16(vt + e0 * 2);
+        vw.q[1] = load16(vt + e1 * 2);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
         union {
           bf16x4_bits v;
-          uint16_t h4[4];
+          uint32_t u[2];
         } va;
-        va.v = load_cache4<FP8>(vt + e * ESZ);
-        // stale bytes past the context may decode to NaN, and 0 * NaN is NaN: those tokens' V is zero
-#pragma unroll
-        for (int r = 0; r < 4; ++r) va.h4[r] = t4 + r < ctx ? va.h4[r] : (uint16_t)0;
+        if constexpr (FP8) {
+          const uint32_t w = vw.u[j] & keep[j];
+          va.u[0] = fp8x2_to_bf16x2(w, false);
+          va.u[1] = fp8x2_to_bf16x2(w, true);
+        } else {
+          va.u[0] = vw.u[2 * j] & keep[2 * j];
+          va.u[1] = vw.u[2 * j + 1] & keep[2 * j + 1];
+        }
         acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va.v, pb[j], acc[db], 0, 0, 0);
       }
     }

@@ -298,11 +298,19 @@ def plan_decode(
             per = -(-max_seq // int(num_sequence_partitions))
             partition_size = -(-per // PARTITION_GRANULE) * PARTITION_GRANULE
         elif head_size != 128:
-            # the generic kernels run one wave per (sequence, partition, kv head, 16-row tile): the shortest partitions
-            # that still leave the launch under a few dozen waves per SIMD
+            # the generic kernels run one wave per (sequence, partition, kv head, 16-row tile), four waves per SIMD
+            # (two at head size 256): the longest partitions of up to 1024 tokens that still give every wave slot a
+            # wave (measured at 64 sequences x 8 kv heads x 4096 tokens: head 64 67 / 61 / 59 us per call at 256 / 512 /
+            # 1024, head 256 207 / 196 / 228 us at 512 / 1024 / 2048), longer ones only to keep the launch under a few
+            # dozen waves per SIMD
+            def waves(ps):
+                return num_seqs * num_kv_heads * -(-ge // 16) * -(-max_seq // ps)
+
+            slots = torch.cuda.get_device_properties(dev).multi_processor_count * 4 * (2 if head_size == 256 else 4)
             partition_size = PARTITION_GRANULE
-            while (num_seqs * num_kv_heads * -(-ge // 16) * -(-max_seq // partition_size) > 32768
-                   and partition_size < 4096):
+            while partition_size < 1024 and waves(2 * partition_size) >= slots:
+                partition_size *= 2
+            while waves(partition_size) > 32768 and partition_size < 4096:
                 partition_size *= 2
         else:
             partition_size = select_partition_size(num_seqs, num_kv_heads, ge, max_seq, block_size, 0,
