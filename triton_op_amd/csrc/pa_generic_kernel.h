@@ -333,12 +333,15 @@ __global__ __launch_bounds__(64) void pa_reduce_generic_kernel(const PaDecodeArg
   const __bf16* tmp = (const __bf16*)a.tmp_output + (int64_t)b * a.stride_tmp_s + (int64_t)h * a.stride_tmp_h +
                       (int64_t)row * a.stride_tmp_g;
   float M = a.sinks ? a.sinks[h * Ge + row] : -INFINITY;  // (the sink takes part in the maximum)
+  // (the loads of four partitions go out together: the loops are round trips to memory otherwise)
+#pragma unroll 4
   for (int p = 0; p < n; ++p) M = fmaxf(M, a.max_logits[es + (int64_t)p * a.stride_es_p]);
   const float M_safe = M == -INFINITY ? 0.f : M;
   float L = 0.f;
   float o[DPL];
 #pragma unroll
   for (int i = 0; i < DPL; ++i) o[i] = 0.f;
+#pragma unroll 4
   for (int p = 0; p < n; ++p) {
     const float w = a.exp_sums[es + (int64_t)p * a.stride_es_p] *
                     __expf(a.max_logits[es + (int64_t)p * a.stride_es_p] - M_safe);
