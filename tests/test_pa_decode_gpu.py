@@ -292,6 +292,40 @@ def test_caller_buffers_strided_inputs_and_twin_entry_point(cuda):
     assert (es[1, :, 1:] == 7.0).all() and (to[1, :, 1:] == 7.0).all()
 
 
+def test_teams_with_strided_caller_buffers_and_output(cuda):
+    """A launch in teams through caller-owned buffers that are not contiguous: partition buffers with a longer
+    partition axis, a query and an output whose rows are 256 elements apart, a block table with a longer row."""
+    import triton_op_amd as T
+
+    batch, hkv, group, P = 50, 8, 8, 8
+    gen = torch.Generator().manual_seed(71)
+    ctx = torch.randint(1, 256 * P + 1, (batch,), generator=gen, dtype=torch.int32)
+    ctx[0], ctx[1] = 256 * P, 200
+    wl = _make(batch=batch, num_q_heads=hkv * group, num_kv_heads=hkv, context_lens=ctx)
+    g = wl.to(cuda)
+    es = torch.full((batch, hkv, P + 3, group), 7.0, device=cuda)[:, :, :P]
+    ml = torch.full((batch, hkv, P + 3, group), 7.0, device=cuda)[:, :, :P]
+    to = torch.full((batch, hkv, P + 1, group, 128), 7.0, dtype=torch.bfloat16, device=cuda)[:, :, :P]
+    qpad = torch.zeros(batch, hkv * group, 256, dtype=torch.bfloat16, device=cuda)
+    qpad[:, :, :128] = g.query
+    opad = torch.full((batch, hkv * group, 256), float("nan"), dtype=torch.bfloat16, device=cuda)
+    out = opad[:, :, :128]
+    bt = torch.zeros(batch, g.block_tables.shape[1] + 5, dtype=torch.int32, device=cuda)
+    bt[:, :g.block_tables.shape[1]] = g.block_tables
+    plan = T.plan_decode(out, qpad[:, :, :128], g.key_cache, g.value_cache, g.context_lens,
+                         bt[:, :g.block_tables.shape[1]], g.softmax_scale, 1, 256 * P, torch.bfloat16, None, g.key_scale,
+                         g.value_scale, 0, None, ml, es, to, partition_size=256)
+    assert "teams of 4 waves, 2 partitions per wave" in plan.launch_info(), plan.launch_info()
+    plan.run()
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.float().cpu(), _oracle(wl).float(), atol=ATOL, rtol=RTOL)
+    assert bool(torch.isnan(opad[:, :, 128:].float()).all())  # nothing written between the output's rows
+    merged = O.reduce_stage(ml.cpu(), es.cpu(), to.float().cpu(), wl.context_lens, 256)
+    torch.testing.assert_close(out.float().cpu(), merged.float(), atol=2e-3, rtol=2e-2)
+    # partitions a sequence does not reach are left untouched (sequence 1 has 200 tokens: 1 partition)
+    assert (es[1, :, 1:] == 7.0).all() and (to[1, :, 1:] == 7.0).all()
+
+
 @pytest.mark.parametrize("q_len", [2, 4])
 def test_fp8_query_with_scales(cuda, q_len):
     """FP8 query with a per-row scale, the reference Gluon entry point's own contract
