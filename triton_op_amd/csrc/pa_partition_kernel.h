@@ -216,8 +216,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     }
   }
   const int row0 = 16 * NT * rt;  // first query row of this workgroup inside its kv-head group
-  const int team_part0 = part;     // TEAM: the workgroup's first partition (0: a team takes the whole axis)
-  if constexpr (TEAM) part += team_wave * span;
+  if constexpr (TEAM) part += team_wave * span;  // (a team's item is the sequence's whole axis: its first partition is 0)
   do {  // the body of one item; `break` leaves it
   if constexpr (TEAM) {
     if (part >= P) break;  // (a wave of the team with no partition left)
@@ -1005,7 +1004,7 @@ void pa_partition_kernel(const PaDecodeArgs a) {
     // output the launch layer does not form teams)
     const bool finished = n_live == 1 && ctx_t > 0;
     char* outp_t = (char*)a.output + ((int64_t)b * a.stride_out_s + (int64_t)h * Ge * a.stride_out_h) * 2;
-    if (!finished && team_part0 == 0) {
+    if (!finished) {
       // A half-wave per row (lane: four head dims), two rows of the tile per wave and pass.  Every lane takes the
       // row's maximum over the partitions, then adds up its four dims with the partitions' weights (the maxima and
       // sums are LDS broadcasts: no lane exchanges, and the reads of an unrolled group are independent).
